@@ -1,0 +1,381 @@
+"""Each kernel alone against its plain reference, at sizes other than the engine's."""
+import math
+
+import pytest
+import torch
+
+import plain_qwen3 as plain
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def kern(dtype):
+    from vosti_amd.kernels import kernels_for
+    return kernels_for(dtype)
+
+
+def tol(dtype):
+    # One rounding to the element type of a value of order 1, plus accumulation differences.
+    return dict(rtol=2e-2, atol=2e-2) if dtype == torch.bfloat16 else dict(rtol=2e-5, atol=2e-5)
+
+
+def rand(shape, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,N,K", [(1, 64, 64), (5, 503, 96), (17, 224, 96), (64, 256, 224), (16, 48, 520),
+                                   (65, 130, 520), (130, 96, 1032), (300, 520, 2056), (8, 40, 4104)])
+def test_gemm(dtype, M, N, K):
+    k = kern(dtype)
+    a, w = rand((M, K), dtype, 1), rand((N, K), dtype, 2, 0.1)
+    ref = (a.double() @ w.double().t()).float()
+    got_t = k.gemm(a.cuda(), w.cuda(), kernel=2)
+    torch.testing.assert_close(got_t.float().cpu(), ref.to(dtype).float(), **tol(dtype))
+    if M <= 64:
+        got_s = k.gemm(a.cuda(), w.cuda(), kernel=1)
+        assert torch.equal(got_s, got_t), "the skinny and the tiled kernel must agree bitwise"
+    # A row of a batch equals the same row alone, bitwise.
+    for r in {0, M // 2, M - 1}:
+        one = k.gemm(a[r:r + 1].cuda(), w.cuda())
+        assert torch.equal(one[0], got_t[r])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gemm_fused_qkv_equals_three(dtype):
+    # The reference holds this bitwise (kernels/tests/runtime/test_qkv_matmul.py:20-34).
+    k = kern(dtype)
+    a = rand((37, 96), dtype, 3).cuda()
+    ws = [rand((n, 96), dtype, 4 + i, 0.1).cuda() for i, n in enumerate((256, 64, 64))]
+    fused = k.gemm(a, torch.cat(ws).contiguous())
+    three = torch.cat([k.gemm(a, w) for w in ws], dim=1)
+    assert torch.equal(fused, three)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gemm_refuses_bad_width(dtype):
+    from vosti_amd.kernels.ops import KernelError
+    k = kern(dtype)
+    with pytest.raises(KernelError, match="multiple"):
+        k.gemm(rand((2, 50), dtype, 0).cuda(), rand((8, 50), dtype, 1).cuda())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,H", [(1, 64), (7, 96), (33, 100), (5, 4104), (3, 17)])
+def test_rmsnorm_and_add(dtype, T, H):
+    k = kern(dtype)
+    x, r, w = rand((T, H), dtype, 1), rand((T, H), dtype, 2), (1 + 0.1 * rand((H,), torch.float32, 3)).to(dtype)
+    eps = 1e-5
+    got = k.rmsnorm(x.cuda(), w.cuda(), eps)
+    torch.testing.assert_close(got.float().cpu(), plain.rms_norm(x, w, eps, dtype), **tol(dtype))
+    res = r.clone().cuda()
+    got = k.add_rmsnorm(x.cuda(), res, w.cuda(), eps)
+    ref_n, ref_r = plain.add_rms_norm(x, r, w, eps, dtype)
+    torch.testing.assert_close(got.float().cpu(), ref_n, **tol(dtype))
+    torch.testing.assert_close(res.float().cpu(), ref_r, **tol(dtype))
+    # Norm weights stored in 32-bit stay so.
+    got32 = k.rmsnorm(x.cuda(), w.float().cuda(), eps)
+    torch.testing.assert_close(got32.float().cpu(), plain.rms_norm(x, w, eps, dtype), **tol(dtype))
+    # Row of a batch == the row alone.
+    assert torch.equal(k.rmsnorm(x[T // 2: T // 2 + 1].cuda(), w.cuda(), eps)[0], k.rmsnorm(x.cuda(), w.cuda(), eps)[T // 2])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rmsnorm_unit_rms(dtype):
+    # With w = 1 and eps = 0 every row has unit RMS, whatever its scale.
+    k = kern(dtype)
+    x = (rand((4, 256), torch.float32, 5) * torch.tensor([[1e-2], [1.0], [30.0], [1e3]])).to(dtype)
+    y = k.rmsnorm(x.cuda(), torch.ones(256, dtype=dtype).cuda(), 0.0).float()
+    torch.testing.assert_close((y * y).mean(dim=1).sqrt().cpu(), torch.ones(4), rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,I", [(3, 128), (9, 224), (2, 101)])
+def test_swiglu(dtype, T, I):
+    k = kern(dtype)
+    gu = rand((T, 2 * I), dtype, 1, 2.0)
+    ref = torch.nn.functional.silu(gu[:, :I].float()) * gu[:, I:].float()
+    torch.testing.assert_close(k.swiglu(gu.cuda()).float().cpu(), ref.to(dtype).float(), **tol(dtype))
+    torch.testing.assert_close(k.swiglu(gu.cuda()).float().cpu(), plain.swiglu(gu, dtype), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embedding_and_gather(dtype):
+    k = kern(dtype)
+    table = rand((503, 100), dtype, 1)
+    ids = torch.tensor([0, 502, 7, 7, 250], dtype=torch.int32)
+    got = k.embedding(table.cuda(), ids.cuda())
+    assert torch.equal(got.cpu(), torch.nn.functional.embedding(ids.long(), table))
+    rows = torch.tensor([4, 0, 2], dtype=torch.int32)
+    assert torch.equal(k.gather_rows(got, rows.cuda()).cpu(), got.cpu()[rows.long()])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_argmax_vectors(dtype):
+    # The reference's vectors: ties, NaN, +-inf (python/tests/test_qwen3_kernel_contracts.py:525-539).
+    k = kern(dtype)
+    rows = torch.tensor([[-3.0, 7.0, 7.0, 2.0], [float("nan"), 5.0, float("nan"), 1.0],
+                         [float("-inf"), float("inf"), 4.0, float("inf")]]).to(dtype)
+    assert k.sample(rows.cuda()).cpu().tolist() == [1, 0, 1] == [plain.argmax_token(r) for r in rows]
+    big = rand((3, 5003), dtype, 2)
+    assert k.sample(big.cuda()).cpu().tolist() == torch.argmax(big.float(), dim=1).tolist()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_temperature_sampling(dtype):
+    k = kern(dtype)
+    V = 1003
+    logits = rand((4, V), dtype, 3, 2.0)
+    temps = torch.tensor([0.7, 1.3, 0.0, 0.7])
+    u = torch.tensor([0.25, 0.9, 0.5, 0.25])
+    got = k.sample(logits.cuda(), temps.cuda(), u.cuda()).cpu().tolist()
+    for r in range(4):
+        if temps[r] == 0:
+            assert got[r] == int(torch.argmax(logits[r].float()))
+            continue
+        p = torch.softmax(logits[r].double() / temps[r].double(), dim=0)
+        cdf = torch.cumsum(p, dim=0)
+        # The drawn token's CDF interval contains u, up to float32 rounding of the running sums.
+        lo = cdf[got[r] - 1] if got[r] > 0 else 0.0
+        assert lo - 1e-4 <= u[r] <= cdf[got[r]] + 1e-4
+    # Independent of the companions in the batch.
+    assert k.sample(logits[3:4].cuda(), temps[3:4].cuda(), u[3:4].cuda()).item() == got[3]
+    assert k.sample(logits[1:2].cuda(), temps[1:2].cuda(), u[1:2].cuda()).item() == got[1]
+    # Temperature -> 0 is greedy; u near 1 stays inside the vocabulary.
+    tiny = k.sample(logits.cuda(), torch.full((4,), 1e-4).cuda(), u.cuda()).cpu().tolist()
+    assert tiny == torch.argmax(logits.float(), dim=1).tolist()
+    edge = k.sample(logits.cuda(), torch.ones(4).cuda(), torch.full((4,), 1 - 2 ** -24).cuda()).cpu()
+    assert ((edge >= 0) & (edge < V)).all()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_random_fill_matches_host(dtype):
+    from vosti_amd.weights.random_init import _init_params, random_tensor_cpu, tensor_seed
+    k = kern(dtype)
+    for init, shape in ((("normal", 0.02), (37, 101)), (("uniform", 0.9, 1.1), (1000,))):
+        host = random_tensor_cpu(5, "some.name", shape, init).to(dtype)
+        dev = torch.empty(shape, dtype=dtype, device="cuda")
+        k.fill_random(dev, tensor_seed(5, "some.name"), *_init_params(init))
+        assert torch.equal(dev.cpu(), host)
+    big = random_tensor_cpu(1, "w", (200000,), ("normal", 0.02))
+    assert abs(big.std().item() - 0.02) < 3e-4 and abs(big.mean().item()) < 2e-4
+
+
+# ------------------------------------------------------------------ qkv_post
+def paged_layout(n_tokens, P, n_pages, seed):
+    """A shuffled assignment of logical pages to physical ones."""
+    g = torch.Generator().manual_seed(seed)
+    need = -(-n_tokens // P)
+    return torch.randperm(n_pages, generator=g)[:need].tolist()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,d,P,rot", [(4, 2, 16, 16, 16), (8, 2, 32, 8, 32), (3, 1, 80, 32, 40), (2, 2, 128, 64, 128)])
+def test_qkv_post(dtype, nq, nkv, d, P, rot):
+    k = kern(dtype)
+    T, eps, max_pos, theta = 21, 1e-5, 64, 1e4
+    qkv = rand((T, (nq + 2 * nkv) * d), dtype, 1)
+    qw, kw = (1 + 0.1 * rand((d,), torch.float32, 2)).to(dtype), (1 + 0.1 * rand((d,), torch.float32, 3)).to(dtype)
+    positions = torch.arange(5, 5 + T, dtype=torch.int32)
+    inv = (1.0 / (theta ** (torch.arange(0, rot, 2, dtype=torch.int64).float() / rot))).cuda()
+    cos, sin = k.rope_tables(inv, max_pos)
+    pcos, psin = plain.rope_tables(max_pos, rot, theta, dtype)
+    torch.testing.assert_close(cos.float().cpu(), pcos, rtol=1e-5, atol=1e-5 if dtype == torch.float32 else 1e-2)
+    n_pages = 9
+    pages = paged_layout(5 + T, P, n_pages, 4)
+    slots = torch.tensor([pages[p // P] * P + p % P for p in positions.tolist()], dtype=torch.int32)
+    slots[3] = -1   # writes nothing
+    kc = torch.full((n_pages, nkv, P, d), 7.0, dtype=dtype).cuda()
+    vc = torch.full((n_pages, nkv, d, P), 7.0, dtype=dtype).cuda()
+    q = k.qkv_post(qkv.cuda(), nq=nq, nkv=nkv, d=d, q_out=None, k_cache=kc, v_cache=vc, page_size=P, q_w=qw.cuda(),
+                   k_w=kw.cuda(), eps=eps, cos=cos, sin=sin, positions=positions.cuda(), slots=slots.cuda())
+    x = qkv.view(T, nq + 2 * nkv, d)
+    ref_q = plain.apply_rope(plain.head_rms_norm(x[:, :nq], qw, eps, dtype), pcos, psin, positions, dtype)
+    ref_k = plain.apply_rope(plain.head_rms_norm(x[:, nq:nq + nkv], kw, eps, dtype), pcos, psin, positions, dtype)
+    torch.testing.assert_close(q.float().cpu(), ref_q, **tol(dtype))
+    kc, vc = kc.cpu(), vc.cpu()
+    written = torch.zeros(n_pages * P, dtype=torch.bool)
+    for t in range(T):
+        s = int(slots[t])
+        if s < 0:
+            continue
+        written[s] = True
+        torch.testing.assert_close(kc[s // P, :, s % P, :].float(), ref_k[t], **tol(dtype))
+        assert torch.equal(vc[s // P, :, :, s % P], x[t, nq + nkv:]), "a stored value row is the input row, bytewise"
+    # Unwritten slots are unchanged.
+    untouched_k = kc.permute(0, 2, 1, 3).reshape(n_pages * P, nkv, d)[~written]
+    assert (untouched_k == 7.0).all()
+    untouched_v = vc.permute(0, 3, 1, 2).reshape(n_pages * P, nkv, d)[~written]
+    assert (untouched_v == 7.0).all()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rope_invariants(dtype):
+    """Position 0 is the identity; a rotation keeps each pair's norm; the product of a
+    rotated q and k depends on the distance of their positions only (float32)."""
+    k = kern(dtype)
+    d, theta, max_pos = 32, 1e4, 128
+    inv = (1.0 / (theta ** (torch.arange(0, d, 2, dtype=torch.int64).float() / d))).cuda()
+    cos, sin = k.rope_tables(inv, max_pos)
+
+    def rot(x, pos):
+        T = x.shape[0]
+        return k.qkv_post(x.view(T, -1), nq=x.shape[1], nkv=0, d=d, q_out=None, k_cache=None, v_cache=None, page_size=0,
+                          q_w=None, k_w=None, eps=0.0, cos=cos, sin=sin,
+                          positions=torch.tensor(pos, dtype=torch.int32).cuda(), slots=None)
+    x = rand((3, 2, d), dtype, 1).cuda()
+    assert torch.equal(rot(x, [0, 0, 0]), x)
+    y = rot(x, [3, 17, 90]).float()
+    xf = x.float()
+    torch.testing.assert_close(y[..., :16] ** 2 + y[..., 16:] ** 2, xf[..., :16] ** 2 + xf[..., 16:] ** 2, **tol(dtype))
+    if dtype == torch.float32:
+        q, kk = rand((1, 1, d), dtype, 2).cuda(), rand((1, 1, d), dtype, 3).cuda()
+        dots = [(rot(q, [p + 9]) * rot(kk, [p])).sum().item() for p in (0, 5, 40, 100)]
+        assert max(dots) - min(dots) < 1e-4
+        # A wrong sign or pairing fails this: the half-rotation form x*cos + rotate_half(x)*sin.
+        pos = [11]
+        c, s = cos[11].float(), sin[11].float()
+        x1, x2 = q[0, 0, :16], q[0, 0, 16:]
+        want = torch.cat([x1 * c - x2 * s, x2 * c + x1 * s])
+        torch.testing.assert_close(rot(q, pos)[0, 0], want, rtol=1e-6, atol=1e-6)
+
+
+# ----------------------------------------------------------------- attention
+def build_cache(kk, vv, P, n_pages, seed, dtype, poison=None):
+    """kk, vv: lists per sequence of [len, nkv, d].  Returns caches, block table and k_len."""
+    nkv, d = kk[0].shape[1:]
+    fill = 0.0 if poison is None else poison
+    kc = torch.full((n_pages, nkv, P, d), fill, dtype=dtype)
+    vc = torch.full((n_pages, nkv, d, P), fill, dtype=dtype)
+    g = torch.Generator().manual_seed(seed)
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    width = max(-(-k.shape[0] // P) for k in kk)
+    table = torch.full((len(kk), width + 1), perm[-1], dtype=torch.int32)   # padded entries: a poisoned page
+    for s, (k, v) in enumerate(zip(kk, vv)):
+        for j in range(-(-k.shape[0] // P)):
+            page = perm.pop(0)
+            table[s, j] = page
+            n = min(P, k.shape[0] - j * P)
+            kc[page, :, :n, :] = k[j * P:j * P + n].permute(1, 0, 2)
+            vc[page, :, :, :n] = v[j * P:j * P + n].permute(1, 2, 0)
+    return kc, vc, table
+
+
+def run_attention(k, q_list, kk, vv, P, dtype, window=0, poison=None, decode_split=None, seed=0):
+    n_pages = sum(-(-x.shape[0] // P) for x in kk) + 3
+    kc, vc, table = build_cache(kk, vv, P, n_pages, seed, dtype, poison)
+    q = torch.cat(q_list).cuda()
+    q_lens = [x.shape[0] for x in q_list]
+    cu = torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32)
+    k_len = torch.tensor([x.shape[0] for x in kk], dtype=torch.int32)
+    out = torch.zeros_like(q)
+    pre = [(s, o) for s, n in enumerate(q_lens) if n > 1 for o in range(0, n, 16)]
+    dec = [(s, 0) for s, n in enumerate(q_lens) if n == 1]
+    d = q.shape[2]
+    args = (q, kc.cuda(), vc.cuda(), table.cuda(), cu.cuda(), k_len.cuda())
+    kw = dict(scale=d ** -0.5, window=window, max_k_len=int(k_len.max()), out=out)
+    if pre:
+        k.paged_attention(*args, torch.tensor(pre, dtype=torch.int32).cuda(), mode=0, **kw)
+    if dec:
+        items = torch.tensor(dec, dtype=torch.int32).cuda()
+        if decode_split:
+            nseg = -(-int(k_len.max()) // 256) + 1
+            scratch = torch.full((k.attn_scratch_floats(q.shape[0], q.shape[1], d, nseg),), float("nan"), device="cuda")
+            k.paged_attention(*args, items, mode=1, split=True, nseg=nseg, scratch=scratch, **kw)
+        else:
+            k.paged_attention(*args, items, mode=1, **kw)
+    return out.cpu()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,d,P", [(4, 2, 16, 16), (8, 2, 32, 8), (6, 1, 80, 32), (4, 4, 128, 64), (20, 1, 48, 16)])
+def test_attention_against_plain(dtype, nq, nkv, d, P):
+    """Lengths straddling pages and tiles (the reference's self-test uses 63/64/65/129 against
+    255/256/257/321: kernels/triton_kernels/fattn_paged.py:893-924), decode rows beside prompt rows,
+    a shuffled page order, and NaN in every unused page, tail and padded table entry."""
+    k = kern(dtype)
+    shapes = [(63, 255), (64, 256), (65, 257), (129, 321), (1, 7), (1, 300), (3, 7), (1, 1), (2, 64), (17, 17)]
+    q_list, kk, vv = [], [], []
+    for i, (ql, kl) in enumerate(shapes):
+        q_list.append(rand((ql, nq, d), dtype, 10 + i))
+        kk.append(rand((kl, nkv, d), dtype, 30 + i))
+        vv.append(rand((kl, nkv, d), dtype, 50 + i))
+    got = run_attention(k, q_list, kk, vv, P, dtype, poison=float("nan"))
+    off = 0
+    for q, kx, vx in zip(q_list, kk, vv):
+        ref = plain.attention(q, kx, vx, d ** -0.5, dtype)
+        torch.testing.assert_close(got[off:off + q.shape[0]].float(), ref, **tol(dtype))
+        off += q.shape[0]
+    # Poison changes nothing bitwise; the split decode path gives the same bits as the fused one.
+    clean = run_attention(k, q_list, kk, vv, P, dtype, poison=None, decode_split=True, seed=5)
+    assert torch.equal(clean, got)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_cutting_is_bitwise_invisible(dtype):
+    """A row's result depends on its own query and its keys only: the same position computed as a
+    prompt row, as a row of a shorter portion, and as a decoded token gives the same bits."""
+    k = kern(dtype)
+    nq, nkv, d, P, L = 8, 2, 64, 16, 600
+    q, kx, vx = rand((L, nq, d), dtype, 1), rand((L, nkv, d), dtype, 2), rand((L, nkv, d), dtype, 3)
+    whole = run_attention(k, [q], [kx], [vx], P, dtype)
+    for start, n in ((L - 1, 1), (300, 1), (255, 2), (250, 37), (0, 1), (511, 5)):
+        part = run_attention(k, [q[start:start + n]], [kx[:start + n]], [vx[:start + n]], P, dtype, decode_split=(n == 1))
+        assert torch.equal(part, whole[start:start + n]), (start, n)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_far_key_and_window(dtype):
+    """One key among hundreds is made to stand out, so that a kernel that loses a far key, a page or
+    a window's edge shows: the output must be that key's value.  Then a window that ends just before
+    or just at that key."""
+    k = kern(dtype)
+    nq, nkv, d, P, L = 4, 2, 32, 8, 700
+    for far in (0, 7, 8, 255, 256, 511, 640):
+        q = rand((1, nq, d), dtype, 1) * 0.1
+        kx, vx = rand((L, nkv, d), dtype, 2) * 0.1, rand((L, nkv, d), dtype, 3)
+        q[0, :, 0] = 40.0
+        kx[far, :, 0] = 40.0       # score 1600 * scale: everything else vanishes
+        got = run_attention(k, [q], [kx], [vx], P, dtype, decode_split=True)
+        want = vx[far].float().repeat_interleave(nq // nkv, dim=0)
+        torch.testing.assert_close(got[0].float(), want, **tol(dtype))
+        # Window: position L-1 sees keys L-window .. L-1.
+        inside = run_attention(k, [q], [kx], [vx], P, dtype, window=L - far)
+        torch.testing.assert_close(inside[0].float(), want, **tol(dtype))
+        if far < L - 1:
+            outside = run_attention(k, [q], [kx], [vx], P, dtype, window=L - far - 1)
+            ref = plain.attention(q, kx, vx, d ** -0.5, dtype, window=L - far - 1)
+            torch.testing.assert_close(outside.float(), ref, **tol(dtype))
+            assert not torch.allclose(outside[0].float(), want, atol=0.05)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_special_cases(dtype):
+    """One head without mask (a single decoded row over all keys) is the library softmax."""
+    k = kern(dtype)
+    d, L = 64, 200
+    q, kx, vx = rand((1, 1, d), dtype, 1), rand((L, 1, d), dtype, 2), rand((L, 1, d), dtype, 3)
+    got = run_attention(k, [q], [kx], [vx], 16, dtype)
+    p = torch.softmax((kx[:, 0].float() @ q[0, 0].float()) * d ** -0.5, dim=0)
+    torch.testing.assert_close(got[0, 0].float(), p @ vx[:, 0].float(), **tol(dtype))
+    # q_len == k_len: plain causal attention through the library routine.
+    q = rand((50, 2, d), dtype, 4)
+    kx, vx = rand((50, 2, d), dtype, 5), rand((50, 2, d), dtype, 6)
+    got = run_attention(k, [q], [kx], [vx], 8, dtype)
+    ref = torch.nn.functional.scaled_dot_product_attention(q.float().transpose(0, 1), kx.float().transpose(0, 1),
+                                                           vx.float().transpose(0, 1), is_causal=True).transpose(0, 1)
+    torch.testing.assert_close(got.float(), ref, **tol(dtype))
+
+
+def test_attention_refuses_bad_sizes():
+    from vosti_amd.kernels.ops import KernelError
+    k = kern(torch.float32)
+    q = torch.zeros(1, 2, 24, device="cuda")
+    kc, vc = torch.zeros(2, 1, 8, 24, device="cuda"), torch.zeros(2, 1, 24, 8, device="cuda")
+    i32 = lambda *v: torch.tensor(v, dtype=torch.int32, device="cuda")
+    with pytest.raises(KernelError, match="head size"):
+        k.paged_attention(q, kc, vc, i32(0, 1).view(1, 2), i32(0, 1), i32(1), i32(0, 0).view(1, 2), mode=1, scale=1.0,
+                          max_k_len=1)

@@ -1,0 +1,63 @@
+"""Loads the native host library (cache manager and scheduler)."""
+from __future__ import annotations
+
+import ctypes
+from ctypes import POINTER, c_char_p, c_int, c_int32, c_int64, c_uint64, c_void_p
+
+from ..kernels import build
+
+ABI_VERSION = 3
+_LIB = None
+
+
+def host_lib():
+    global _LIB
+    if _LIB is not None:
+        return _LIB
+    lib = ctypes.CDLL(str(build.ensure("host")))
+    lib.vh_abi_version.restype = c_int
+    if lib.vh_abi_version() != ABI_VERSION:
+        raise RuntimeError("libvosti_host.so is stale; rebuild it")
+    I, U, P = c_int, c_uint64, c_void_p
+    PI = POINTER(c_int32)
+
+    def sig(name, restype, *args):
+        fn = getattr(lib, name)
+        fn.restype, fn.argtypes = restype, list(args)
+
+    sig("vh_cache_create", P, I, I, POINTER(c_int), POINTER(c_int), I, I)
+    sig("vh_cache_destroy", None, P)
+    sig("vh_cache_add_request", I, P, U, PI, I, POINTER(c_int))
+    sig("vh_cache_reserve", I, P, U, I)
+    sig("vh_cache_extend", I, P, U, PI, I)
+    for n in ("commit", "abort_step", "finish", "has_request", "length", "pending", "state_slot"):
+        sig(f"vh_cache_{n}", I, P, U)
+    sig("vh_cache_num_logical_pages", I, P, U, I)
+    sig("vh_cache_available_pages", I, P, I)
+    sig("vh_cache_free_pages", I, P, I)
+    for n in ("free_slots", "num_requests", "cached_blocks"):
+        sig(f"vh_cache_{n}", I, P)
+    sig("vh_cache_prefix_hits", c_int64, P)
+    sig("vh_cache_evictions", c_int64, P)
+    sig("vh_cache_fill_block_table", I, P, U, I, c_void_p, I)
+    sig("vh_cache_fill_slots", I, P, U, I, I, I, c_void_p)
+    sig("vh_cache_check", I, P, c_char_p, I)
+    sig("vh_sched_create", P, P, I, I, I)
+    sig("vh_sched_destroy", None, P)
+    sig("vh_sched_add_request", I, P, U, PI, I, I, PI, I, I)
+    sig("vh_sched_plan", I, P, POINTER(c_int), POINTER(c_int))
+    sig("vh_sched_get_plan", None, P, c_void_p, c_void_p)
+    sig("vh_sched_commit", I, P, PI, I)
+    sig("vh_sched_get_emitted", None, P, c_void_p)
+    sig("vh_sched_abort", I, P, U)
+    sig("vh_sched_num_waiting", I, P)
+    sig("vh_sched_num_running", I, P)
+    sig("vh_sched_preemptions", c_int64, P)
+    sig("vh_sched_is_live", I, P, U)
+    _LIB = lib
+    return lib
+
+
+def i32_array(values):
+    arr = (c_int32 * len(values))(*values)
+    return arr

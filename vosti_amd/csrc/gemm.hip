@@ -1,0 +1,299 @@
+// out[M,N] = act[M,K] * w[N,K]^T  (weights in [out_features, in_features] layout).
+//
+// Reduction order, the same in every kernel of this file and for every M:
+//   K is cut into chunks of 512 elements starting at 0.  Within a chunk the
+//   products are accumulated from zero by mma_slab() over the chunk's slabs in
+//   ascending order (weights are the first MFMA operand, activations the
+//   second).  The chunk sums are then added to a zero total in ascending chunk
+//   order, and the total is rounded to the element type once.
+// An output element therefore never depends on M, on the other rows of its
+// tile or on which kernel produced it; the choice between the kernels is a
+// matter of speed only.  The reference keys its tile configuration on (N, K)
+// for the same reason (kernels/triton_kernels/matmul.py:33-73,
+// kernels/triton_kernels/qkv_matmul.py:24-32).
+//
+//   gemm_skinny: M <= 64.  Streams the weights once from HBM; a workgroup of
+//                eight waves owns 16*NTW weight rows and the waves split K by
+//                chunk.  Chunk sums meet in LDS and are added in chunk order.
+//   gemm_tiled:  any M.  128x128 output tile per workgroup staged through LDS,
+//                64x64 per wave; a second accumulator set holds the total.
+#include "common.h"
+#include "mma.h"
+#include "vec.h"
+
+#define KC 512                        // elements per chunk
+#define KC_SLABS (KC / VK_SLAB)       // 16 (bfloat16) or 32 (float)
+
+__device__ __forceinline__ void store_out4(elem_t* out, int64_t ldo, int m, int n, int M, int N, f32x4 v,
+                                           bool vec_ok) {
+  if (m >= M || n >= N) return;
+  elem_t* p = out + (int64_t)m * ldo + n;
+  if (vec_ok && n + 3 < N) {
+#ifdef VK_F32
+    *reinterpret_cast<f32x4*>(p) = v;
+#else
+    bf16x4 o;
+    o[0] = (__bf16)v.x; o[1] = (__bf16)v.y; o[2] = (__bf16)v.z; o[3] = (__bf16)v.w;
+    *reinterpret_cast<bf16x4*>(p) = o;
+#endif
+  } else {
+    p[0] = from_f32<elem_t>(v.x);
+    if (n + 1 < N) p[1] = from_f32<elem_t>(v.y);
+    if (n + 2 < N) p[2] = from_f32<elem_t>(v.z);
+    if (n + 3 < N) p[3] = from_f32<elem_t>(v.w);
+  }
+}
+
+// ------------------------------------------------------------------ skinny
+template <int NTW, int MT>
+__global__ __launch_bounds__(512) void gemm_skinny_kernel(elem_t* __restrict__ out, const elem_t* __restrict__ act,
+                                                          const elem_t* __restrict__ w, int M, int N, int K,
+                                                          int64_t lda, int64_t ldo, int out_vec_ok) {
+  constexpr int ITEMS = NTW * MT;
+  constexpr int SL = 16 / NTW;            // slabs per stage (a stage is 16 weight fragments)
+  constexpr int NST = KC_SLABS / SL;      // stages per chunk
+  __shared__ f32x4 part[8][ITEMS][64];
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r16 = lane & 15, kg = lane >> 4;
+  const int n0 = blockIdx.x * (16 * NTW);
+  const int nchunks = (K + KC - 1) / KC;
+  const int rounds = (nchunks + 7) / 8;
+
+  const elem_t* wrow[NTW];
+  bool wok[NTW];
+#pragma unroll
+  for (int nt = 0; nt < NTW; ++nt) {
+    const int n = n0 + nt * 16 + r16;
+    wok[nt] = n < N;
+    wrow[nt] = w + (int64_t)(wok[nt] ? n : 0) * K;
+  }
+  const elem_t* arow[MT];
+  bool aok[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = mt * 16 + r16;
+    aok[mt] = m < M;
+    arow[mt] = act + (int64_t)(aok[mt] ? m : 0) * lda;
+  }
+
+  f32x4 total = {0.f, 0.f, 0.f, 0.f};
+
+  for (int round = 0; round < rounds; ++round) {
+    const int c = round * 8 + wave;
+    f32x4 acc[NTW][MT];
+#pragma unroll
+    for (int nt = 0; nt < NTW; ++nt)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    if (c < nchunks) {
+      const int kbase = c * KC + kg * VK_VEC;
+      frag_t cur[16], nxt[16];
+#pragma unroll
+      for (int sl = 0; sl < SL; ++sl)
+#pragma unroll
+        for (int nt = 0; nt < NTW; ++nt) {
+          const int k = kbase + sl * VK_SLAB;
+          cur[sl * NTW + nt] = load_frag(wrow[nt] + k, wok[nt] && k < K);
+        }
+#pragma unroll
+      for (int st = 0; st < NST; ++st) {
+        if (st + 1 < NST) {
+#pragma unroll
+          for (int sl = 0; sl < SL; ++sl)
+#pragma unroll
+            for (int nt = 0; nt < NTW; ++nt) {
+              const int k = kbase + ((st + 1) * SL + sl) * VK_SLAB;
+              nxt[sl * NTW + nt] = load_frag(wrow[nt] + k, wok[nt] && k < K);
+            }
+        }
+#pragma unroll
+        for (int sl = 0; sl < SL; ++sl) {
+          const int k = kbase + (st * SL + sl) * VK_SLAB;
+          frag_t af[MT];
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) af[mt] = load_frag(arow[mt] + k, aok[mt] && k < K);
+#pragma unroll
+          for (int nt = 0; nt < NTW; ++nt)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = mma_slab(cur[sl * NTW + nt], af[mt], acc[nt][mt]);
+        }
+        if (st + 1 < NST) {
+#pragma unroll
+          for (int i = 0; i < 16; ++i) cur[i] = nxt[i];
+        }
+      }
+    }
+#pragma unroll
+    for (int nt = 0; nt < NTW; ++nt)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) part[wave][nt * MT + mt][lane] = acc[nt][mt];
+    __syncthreads();
+    if (wave < ITEMS) {
+      for (int w2 = 0; w2 < 8; ++w2) {
+        if (round * 8 + w2 < nchunks) {
+          const f32x4 p = part[w2][wave][lane];
+          total.x = total.x + p.x; total.y = total.y + p.y; total.z = total.z + p.z; total.w = total.w + p.w;
+        }
+      }
+    }
+    __syncthreads();
+  }
+  if (wave < ITEMS) {
+    const int nt = wave / MT, mt = wave - nt * MT;
+    store_out4(out, ldo, mt * 16 + r16, n0 + nt * 16 + 4 * kg, M, N, total, out_vec_ok);
+  }
+}
+
+// ------------------------------------------------------------------- tiled
+#define T_BM 128
+#define T_BN 128
+#define T_ROWB 128                     // LDS bytes per tile row: two slabs; 16-byte columns are XOR-swizzled by row
+#define T_TILE_BYTES (128 * T_ROWB)
+#define T_CHUNK_TILES (KC_SLABS / 2)   // K tiles (of two slabs) per chunk
+
+__global__ __launch_bounds__(256) void gemm_tiled_kernel(elem_t* __restrict__ out, const elem_t* __restrict__ act,
+                                                         const elem_t* __restrict__ w, int M, int N, int K,
+                                                         int64_t lda, int64_t ldo, int out_vec_ok) {
+  __shared__ __attribute__((aligned(16))) unsigned char lds[2][2][T_TILE_BYTES];  // [buffer][0: w, 1: act]
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r16 = lane & 15, kg = lane >> 4;
+  const int wn = wave & 1, wm = wave >> 1;
+  const int n_blk = blockIdx.x * T_BN, m_blk = blockIdx.y * T_BM;
+  const int nslabs = (K + VK_SLAB - 1) / VK_SLAB;
+  const int ntiles = (nslabs + 1) / 2;
+
+  // Global -> LDS mapping: thread loads 16 bytes at column c16 of rows lrow + 32*i.
+  const int lrow = tid >> 3, c16 = tid & 7;
+  const elem_t* gw[4];
+  const elem_t* ga[4];
+  bool gw_ok[4], ga_ok[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int n = n_blk + lrow + 32 * i, m = m_blk + lrow + 32 * i;
+    gw_ok[i] = n < N;
+    ga_ok[i] = m < M;
+    gw[i] = w + (int64_t)(gw_ok[i] ? n : 0) * K + c16 * VK_VEC;
+    ga[i] = act + (int64_t)(ga_ok[i] ? m : 0) * lda + c16 * VK_VEC;
+  }
+
+  frag_t rw[4], ra[4];
+  auto gload = [&](int kt) {
+    const int k = kt * 2 * VK_SLAB;
+    const bool kok = k + c16 * VK_VEC < K;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      rw[i] = load_frag(gw[i] + k, gw_ok[i] && kok);
+      ra[i] = load_frag(ga[i] + k, ga_ok[i] && kok);
+    }
+  };
+  auto lstore = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int off = (lrow + 32 * i) * T_ROWB + ((c16 ^ (lrow & 7)) * 16);
+      *reinterpret_cast<frag_t*>(&lds[buf][0][off]) = rw[i];
+      *reinterpret_cast<frag_t*>(&lds[buf][1][off]) = ra[i];
+    }
+  };
+
+  f32x4 acc[4][4], total[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+      total[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+
+  gload(0);
+  lstore(0);
+  __syncthreads();
+
+  for (int kt = 0; kt < ntiles; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < ntiles) gload(kt + 1);
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      frag_t wf[4], af[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int col = ((s * 4 + kg) ^ (r16 & 7)) * 16;
+        wf[i] = *reinterpret_cast<const frag_t*>(&lds[buf][0][(wn * 64 + i * 16 + r16) * T_ROWB + col]);
+        af[i] = *reinterpret_cast<const frag_t*>(&lds[buf][1][(wm * 64 + i * 16 + r16) * T_ROWB + col]);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = mma_slab(wf[i], af[j], acc[i][j]);
+    }
+    if ((kt + 1) % T_CHUNK_TILES == 0 || kt + 1 == ntiles) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          total[i][j].x = total[i][j].x + acc[i][j].x;
+          total[i][j].y = total[i][j].y + acc[i][j].y;
+          total[i][j].z = total[i][j].z + acc[i][j].z;
+          total[i][j].w = total[i][j].w + acc[i][j].w;
+          acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+    }
+    if (kt + 1 < ntiles) lstore(buf ^ 1);
+    __syncthreads();
+  }
+
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      store_out4(out, ldo, m_blk + wm * 64 + j * 16 + r16, n_blk + wn * 64 + i * 16 + 4 * kg, M, N, total[i][j],
+                 out_vec_ok);
+}
+
+// ==================================================================== host
+template <int NTW, int MT>
+static void launch_skinny(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K, int64_t lda,
+                          int64_t ldo, int vec_ok, hipStream_t st) {
+  const int per = 16 * NTW;
+  gemm_skinny_kernel<NTW, MT><<<(N + per - 1) / per, 512, 0, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok);
+}
+
+extern "C" {
+
+// kernel: 0 = choose by M, 1 = skinny (M <= 64), 2 = tiled.  The result does not
+// depend on the choice.
+int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K, int64_t lda, int64_t ldo,
+            int kernel, hipStream_t st) {
+  VK_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
+  VK_REQUIRE(K % VK_VEC == 0, "gemm: K=%d must be a multiple of %d for this element type", K, VK_VEC);
+  VK_REQUIRE(K <= 8 * 8 * KC, "gemm: K=%d exceeds the supported maximum of %d", K, 8 * 8 * KC);
+  VK_REQUIRE(lda >= K && lda % VK_VEC == 0, "gemm: activation row stride %lld must be >= K and a multiple of %d",
+             (long long)lda, VK_VEC);
+  VK_REQUIRE(ldo >= N, "gemm: output row stride %lld is smaller than N=%d", (long long)ldo, N);
+  VK_REQUIRE(((uintptr_t)act % 16) == 0 && ((uintptr_t)w % 16) == 0, "gemm: operands must be 16-byte aligned");
+  VK_REQUIRE(kernel >= 0 && kernel <= 2, "gemm: unknown kernel %d", kernel);
+  if (M == 0) return 0;
+  const int vec_ok = (ldo % 4 == 0) && ((uintptr_t)out % 16 == 0);
+  if (kernel == 0) kernel = M <= 64 ? 1 : 2;
+  if (kernel == 1) {
+    VK_REQUIRE(M <= 64, "gemm: the skinny kernel takes at most 64 rows, got %d", M);
+    const int mt = (M + 15) / 16;
+    int ntw = N >= 65536 ? 4 : (N >= 16384 ? 2 : 1);
+    while (ntw * mt > 4) ntw >>= 1;
+#define SK(NTW, MT) launch_skinny<NTW, MT>(out, act, w, M, N, K, lda, ldo, vec_ok, st)
+    if (mt == 1) { if (ntw == 4) SK(4, 1); else if (ntw == 2) SK(2, 1); else SK(1, 1); }
+    else if (mt == 2) { if (ntw == 2) SK(2, 2); else SK(1, 2); }
+    else if (mt == 3) SK(1, 3);
+    else SK(1, 4);
+#undef SK
+    return vk_check_launch("gemm_skinny");
+  }
+  dim3 grid((N + T_BN - 1) / T_BN, (M + T_BM - 1) / T_BM);
+  VK_REQUIRE(grid.y <= 65535, "gemm: too many rows (%d)", M);
+  gemm_tiled_kernel<<<grid, 256, 0, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok);
+  return vk_check_launch("gemm_tiled");
+}
+
+}  // extern "C"

@@ -1,0 +1,139 @@
+// What happens to the q, k and v rows between the QKV projection and attention,
+// in one launch: per-head RMSNorm of q and k, rotary position encoding of q and
+// k, and the write of k and v into their pages.  Each step is optional, so the
+// same kernel also serves as a plain head norm, a plain rotation or a plain
+// cache store.
+//
+// Formulas (reference):
+//   head norm  kernels/triton_kernels/qk_norm.py:67-95   y = x*rsqrt(mean(x^2)+eps)*w, rounded
+//   rotation   kernels/triton_kernels/rope.py:78-123     y1 = x1*cos - x2*sin; y2 = x2*cos + x1*sin,
+//              halves split at rot/2, on the rounded norm output, tables indexed by position
+//   store      kernels/triton_kernels/store_kv_cache.py:89-120   slot -1 writes nothing
+// The reference runs them as five launches (src/exec/dense_swiglu_decoder.rs:207-272).
+//
+// One wave per (token, head); lane l owns elements l, l+64, l+128, l+192.
+#include "common.h"
+#include "vec.h"
+
+struct QkvPostArgs {
+  const elem_t* qkv;      // [T, row_stride]: nq q heads, then nkv k heads, then nkv v heads, d each
+  int64_t row_stride;
+  elem_t* q_out;          // [T, nq, d]
+  elem_t* kc;             // [pages, nkv, P, d]
+  elem_t* vc;             // [pages, nkv, d, P]
+  const void* q_w;        // [d] or null
+  const void* k_w;        // [d] or null
+  const elem_t* cos_t;    // [max_pos, rot_half] or null
+  const elem_t* sin_t;
+  const int32_t* positions;  // [T]
+  const int32_t* slots;      // [T]: page * P + offset, or -1
+  int w_is_f32, nq, nkv, d, P, rot_half;
+  float eps;
+};
+
+__global__ __launch_bounds__(64) void qkv_post_kernel(QkvPostArgs a) {
+  __shared__ float y[256];
+  const int tok = blockIdx.x, hh = blockIdx.y, lane = threadIdx.x;
+  const int d = a.d;
+  const int kind = hh < a.nq ? 0 : (hh < a.nq + a.nkv ? 1 : 2);   // q, k, v
+  const elem_t* x = a.qkv + tok * a.row_stride + (int64_t)hh * d;
+  const void* w = kind == 0 ? a.q_w : (kind == 1 ? a.k_w : nullptr);
+
+  float xv[4];
+  float part = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int c = lane + 64 * i;
+    xv[i] = c < d ? to_f32(x[c]) : 0.f;
+    part = part + xv[i] * xv[i];
+  }
+  if (w != nullptr) {
+    const float total = wave_sum_xor(part);
+    const float rr = rsqrtf(total / (float)d + a.eps);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = lane + 64 * i;
+      if (c < d) xv[i] = round_to_elem((xv[i] * rr) * load_weight(w, a.w_is_f32, c));
+    }
+  }
+  const bool rotate = a.cos_t != nullptr && kind != 2;
+  if (rotate) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = lane + 64 * i;
+      if (c < d) y[c] = xv[i];
+    }
+    __syncthreads();
+    const int rh = a.rot_half;
+    const int64_t trow = (int64_t)a.positions[tok] * rh;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = lane + 64 * i;
+      if (c < rh) {
+        const float cs = to_f32(a.cos_t[trow + c]), sn = to_f32(a.sin_t[trow + c]);
+        xv[i] = y[c] * cs - y[c + rh] * sn;
+      } else if (c < 2 * rh) {
+        const float cs = to_f32(a.cos_t[trow + c - rh]), sn = to_f32(a.sin_t[trow + c - rh]);
+        xv[i] = y[c] * cs + y[c - rh] * sn;
+      }
+    }
+  }
+  if (kind == 0) {
+    elem_t* o = a.q_out + ((int64_t)tok * a.nq + hh) * d;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = lane + 64 * i;
+      if (c < d) o[c] = from_f32<elem_t>(xv[i]);
+    }
+    return;
+  }
+  const int slot = a.slots[tok];
+  if (slot < 0) return;
+  const int page = slot / a.P, off = slot - page * a.P;
+  if (kind == 1) {
+    const int kh = hh - a.nq;
+    elem_t* o = a.kc + (((int64_t)page * a.nkv + kh) * a.P + off) * d;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = lane + 64 * i;
+      if (c < d) o[c] = from_f32<elem_t>(xv[i]);
+    }
+  } else {
+    const int kh = hh - a.nq - a.nkv;
+    elem_t* o = a.vc + ((int64_t)page * a.nkv + kh) * d * a.P + off;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = lane + 64 * i;
+      if (c < d) o[(int64_t)c * a.P] = from_f32<elem_t>(xv[i]);
+    }
+  }
+}
+
+extern "C" {
+
+// Null q_w / k_w: no norm for that kind.  Null cos_t: no rotation.  nkv == 0:
+// only q rows (a plain norm and/or rotation of [T, nq, d]).  nq == 0: only the
+// store.  Positions must lie below the tables' row count and slots inside the
+// cache; the caller checks both on the host before the upload.
+int vk_qkv_post(const elem_t* qkv, int64_t row_stride, elem_t* q_out, elem_t* kc, elem_t* vc, const void* q_w,
+                const void* k_w, int w_is_f32, const elem_t* cos_t, const elem_t* sin_t, int rot_half,
+                const int32_t* positions, const int32_t* slots, int T, int nq, int nkv, int d, int P, float eps,
+                hipStream_t st) {
+  VK_REQUIRE(T >= 0 && nq >= 0 && nkv >= 0 && nq + nkv > 0, "qkv_post: bad sizes T=%d nq=%d nkv=%d", T, nq, nkv);
+  VK_REQUIRE(d > 0 && d <= 256, "qkv_post: head size %d must be in 1..256", d);
+  VK_REQUIRE(row_stride >= (int64_t)(nq + 2 * nkv) * d, "qkv_post: row stride %lld too small", (long long)row_stride);
+  VK_REQUIRE(cos_t == nullptr || (rot_half > 0 && 2 * rot_half <= d), "qkv_post: rotary width %d does not fit head size %d",
+             2 * rot_half, d);
+  VK_REQUIRE(cos_t == nullptr || positions != nullptr, "qkv_post: rotation needs positions");
+  VK_REQUIRE(nkv == 0 || (slots != nullptr && kc != nullptr && vc != nullptr && P > 0), "qkv_post: store needs slots and caches");
+  VK_REQUIRE(nq + 2 * nkv <= 65535, "qkv_post: too many heads");
+  if (T == 0) return 0;
+  QkvPostArgs a;
+  a.qkv = qkv; a.row_stride = row_stride; a.q_out = q_out; a.kc = kc; a.vc = vc; a.q_w = q_w; a.k_w = k_w;
+  a.cos_t = cos_t; a.sin_t = sin_t; a.positions = positions; a.slots = slots; a.w_is_f32 = w_is_f32;
+  a.nq = nq; a.nkv = nkv; a.d = d; a.P = P; a.rot_half = rot_half; a.eps = eps;
+  qkv_post_kernel<<<dim3(T, nq + 2 * nkv), 64, 0, st>>>(a);
+  return vk_check_launch("qkv_post");
+}
+
+}  // extern "C"

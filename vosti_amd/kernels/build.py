@@ -1,0 +1,160 @@
+"""Compiles the native libraries in-tree.
+
+Three shared libraries are built from ``vosti_amd/csrc``:
+
+* ``libvosti_bf16.so`` and ``libvosti_f32.so``: the gfx950 kernels, the same
+  sources compiled with ``-DVK_BF16`` or ``-DVK_F32`` (hipcc);
+* ``libvosti_host.so``: the cache manager and the scheduler (g++, no GPU code).
+
+A library is rebuilt when the hash of its sources, headers and flags differs
+from the one recorded beside it.  ``ensure()``
+builds only the library that is asked for, so a first call compiles what the
+chosen precision needs and nothing else; it prints a line per compiled file so
+that a long first build is visibly alive.
+"""
+from __future__ import annotations
+
+import hashlib
+import os
+import shutil
+import subprocess
+import sys
+import tempfile
+import time
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+PACKAGE_DIR = Path(__file__).resolve().parent.parent
+CSRC = PACKAGE_DIR / "csrc"
+GPU_ARCH = "gfx950"
+GPU_LIBS = {"bf16": "VK_BF16", "f32": "VK_F32"}
+
+HIPCC_FLAGS = [
+    f"--offload-arch={GPU_ARCH}",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-ffp-contract=off",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall", "-Wextra"]
+
+
+def _writable_dir(preferred: Path, fallback_name: str) -> Path:
+    try:
+        preferred.mkdir(parents=True, exist_ok=True)
+        probe = preferred / f".probe{os.getpid()}"
+        probe.write_text("")
+        probe.unlink()
+        return preferred
+    except OSError:
+        d = Path(tempfile.gettempdir()) / f"vosti_amd_{os.getuid()}" / fallback_name
+        d.mkdir(parents=True, exist_ok=True)
+        return d
+
+
+def lib_dir() -> Path:
+    return _writable_dir(PACKAGE_DIR / "_lib", "lib")
+
+
+def build_dir() -> Path:
+    return _writable_dir(PACKAGE_DIR.parent / "_build", "build")
+
+
+def lib_path(name: str) -> Path:
+    """Path of a built library: the in-tree one if present, else the fallback location."""
+    in_tree = PACKAGE_DIR / "_lib" / f"libvosti_{name}.so"
+    if in_tree.exists():
+        return in_tree
+    return lib_dir() / f"libvosti_{name}.so"
+
+
+def _sources(name: str) -> tuple[list[Path], list[Path]]:
+    if name == "host":
+        return sorted((CSRC / "host").glob("*.cpp")), sorted((CSRC / "host").glob("*.h"))
+    return sorted(CSRC.glob("*.hip")), sorted(CSRC.glob("*.h"))
+
+
+def source_hash(name: str) -> str:
+    srcs, hdrs = _sources(name)
+    h = hashlib.sha256()
+    h.update(repr((HOST_FLAGS if name == "host" else HIPCC_FLAGS + [GPU_LIBS[name]])).encode())
+    for p in srcs + hdrs:
+        h.update(p.name.encode())
+        h.update(p.read_bytes())
+    return h.hexdigest()
+
+
+def is_current(name: str) -> bool:
+    lib = lib_path(name)
+    stamp = Path(str(lib) + ".srchash")
+    return lib.exists() and stamp.exists() and stamp.read_text().strip() == source_hash(name)
+
+
+def _find(tool: str, *candidates: str) -> str:
+    for c in (shutil.which(tool), *candidates):
+        if c and os.path.exists(c):
+            return c
+    raise RuntimeError(f"{tool} not found; it is needed to compile vosti_amd's native code")
+
+
+def _run(cmd: list[str], what: str) -> None:
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"compiling {what} failed:\n{' '.join(cmd)}\n{proc.stdout}")
+
+
+def build(name: str, verbose: bool = True) -> Path:
+    """Compile library ``name`` ('bf16', 'f32' or 'host') unconditionally."""
+    srcs, _ = _sources(name)
+    if not srcs:
+        raise RuntimeError(f"no sources for library {name!r} under {CSRC}")
+    obj_dir = build_dir() / name
+    obj_dir.mkdir(parents=True, exist_ok=True)
+    if name == "host":
+        compiler, flags = _find("g++", "/usr/bin/g++"), HOST_FLAGS
+    else:
+        compiler = _find("hipcc", "/opt/rocm/bin/hipcc")
+        flags = HIPCC_FLAGS + [f"-D{GPU_LIBS[name]}"]
+    t0 = time.time()
+
+    def compile_one(src: Path) -> Path:
+        obj = obj_dir / (src.stem + ".o")
+        _run([compiler, *flags, "-I", str(src.parent), "-c", str(src), "-o", str(obj)], src.name)
+        if verbose:
+            print(f"[vosti_amd build] {name}: compiled {src.name} ({time.time() - t0:.0f}s)", file=sys.stderr, flush=True)
+        return obj
+
+    workers = max(1, min(len(srcs), int(os.environ.get("MAX_JOBS", os.cpu_count() or 4)), 16))
+    with ThreadPoolExecutor(workers) as pool:
+        objs = list(pool.map(compile_one, srcs))
+    out = lib_dir() / f"libvosti_{name}.so"
+    tmp = out.with_suffix(f".tmp{os.getpid()}.so")
+    link = [compiler, "-shared", "-fPIC", "-o", str(tmp), *map(str, objs)]
+    if name != "host":
+        link.insert(1, f"--offload-arch={GPU_ARCH}")
+    _run(link, out.name)
+    os.replace(tmp, out)
+    Path(str(out) + ".srchash").write_text(source_hash(name) + "\n")
+    if verbose:
+        print(f"[vosti_amd build] {name}: linked {out} ({time.time() - t0:.0f}s)", file=sys.stderr, flush=True)
+    return out
+
+
+def ensure(name: str, verbose: bool = True) -> Path:
+    """Return the path of an up-to-date library, compiling it if needed."""
+    if is_current(name):
+        return lib_path(name)
+    if verbose:
+        print(f"[vosti_amd build] {name}: compiling native code (first use)", file=sys.stderr, flush=True)
+    return build(name, verbose)
+
+
+def build_all(verbose: bool = True) -> None:
+    for name in ("host", "bf16", "f32"):
+        build(name, verbose)
+
+
+if __name__ == "__main__":
+    build_all()

@@ -1,0 +1,3 @@
+from .decoder import DecoderModel, build_model
+
+__all__ = ["DecoderModel", "build_model"]
