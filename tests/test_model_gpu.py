@@ -1,0 +1,216 @@
+"""The engine against the plain implementation, under every way of cutting the work."""
+import json
+import os
+import random
+import subprocess
+import sys
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import ROOT, TINY
+from plain_qwen3 import PlainQwen3
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+# float32: only summation order and the last bit of exp / rsqrt differ.
+# bfloat16: the plain implementation rounds where the engine does, but a sum taken in another
+# order can land on the neighbouring bfloat16 (2^-8 relative), and layers carry that on.
+TOL = {"float32": dict(rtol=1e-4, atol=2e-5), "bfloat16": dict(rtol=3e-2, atol=3e-2)}
+LENGTHS = {"A": [1, 7, 33, 64, 100, 128], "B": [2, 17, 63, 65, 120, 129, 200, 256]}
+
+
+def prompts_for(name):
+    rng = random.Random(ord(name) + 11)
+    vocab = TINY[name][0]["vocab_size"]
+    return [[rng.randrange(vocab) for _ in range(n)] for n in LENGTHS[name]]
+
+
+@pytest.fixture(scope="module")
+def plain_logits(tiny_dirs):
+    """Plain logits of every prompt, per configuration and type, computed once."""
+    cache = {}
+
+    def get(name, dtype_name):
+        key = (name, dtype_name)
+        if key not in cache:
+            model = PlainQwen3(tiny_dirs[name], DTYPES[dtype_name])
+            cache[key] = [model.logits(p) for p in prompts_for(name)]
+        return cache[key]
+    return get
+
+
+def make_runner(model_dir, dtype_name, page_size, num_pages, num_slots=8):
+    from vosti_amd.cache import CachePool
+    from vosti_amd.engine import ModelRunner
+    from vosti_amd.models import load_model
+    model = load_model(model_dir, dtype_name)
+    return ModelRunner(model, CachePool(model, page_size=page_size, num_pages=num_pages, num_slots=num_slots))
+
+
+def replay(runner, steps):
+    """steps: list of (entries [(rid, tokens, want)], end [rid]) -> {(rid, position): float32 logits row}."""
+    from vosti_amd.engine import StepEntry
+    out, fed = {}, {}
+    for entries, end in steps:
+        logits = runner.kernels.to_f32(runner.step([StepEntry(r, t, w) for r, t, w in entries])).cpu()
+        row = 0
+        for r, t, w in entries:
+            base = fed.get(r, 0)
+            for place in w:
+                out[(r, base + place)] = logits[row]
+                row += 1
+            fed[r] = base + len(t)
+        for r in end:
+            runner.finish(r)
+            fed.pop(r, None)
+    assert runner.cache.num_requests() == 0 and runner.cache.check() == ""
+    return out
+
+
+def cut_whole(prompts):
+    return [([(i, p, list(range(len(p))))], [i]) for i, p in enumerate(prompts)]
+
+
+def cut_tail(prompts, tail=32):
+    steps = []
+    for i, p in enumerate(prompts):
+        head = max(1, len(p) - tail)
+        steps.append(([(i, p[:head], list(range(head)))], []))
+        for j in range(head, len(p)):
+            steps.append(([(i, p[j:j + 1], [0])], []))
+        steps[-1][1].append(i)
+    return steps
+
+
+def cut_chunks(prompts, sizes=(7, 2, 33, 16, 5, 2, 64, 3, 1, 31)):
+    steps, k = [], 0
+    for i, p in enumerate(prompts):
+        pos = 0
+        while pos < len(p):
+            n = min(sizes[k % len(sizes)], len(p) - pos)
+            k += 1
+            steps.append(([(i, p[pos:pos + n], list(range(n)))], []))
+            pos += n
+        steps[-1][1].append(i)
+    return steps
+
+
+def cut_mixed(prompts, page, max_live=4, seed=5):
+    """Up to four live requests, portions of some beside single tokens of others; returns the
+    steps and the pool size (pages) that just holds the largest set of live requests."""
+    rng = random.Random(seed)
+    order = list(range(len(prompts)))
+    rng.shuffle(order)
+    waiting, live, pos, steps = order[:], [], {}, []
+    peak = 0
+    while waiting or live:
+        while waiting and len(live) < max_live:
+            r = waiting.pop(0)
+            live.append(r)
+            pos[r] = 0
+        peak = max(peak, sum(-(-len(prompts[r]) // page) for r in live))
+        entries, end = [], []
+        for r in list(live):
+            if rng.random() < 0.2 and len(live) > 1:
+                continue                       # left out of this step, goes on later
+            left = len(prompts[r]) - pos[r]
+            n = min(left, rng.choice([1, 1, 1, 2, 3, 9, 16, 40]))
+            entries.append((r, prompts[r][pos[r]:pos[r] + n], list(range(n))))
+            pos[r] += n
+            if pos[r] == len(prompts[r]):
+                end.append(r)
+                live.remove(r)
+        if entries:
+            steps.append((entries, end))
+    return steps, peak
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_every_cutting(tiny_dirs, plain_logits, name, dtype_name):
+    prompts = prompts_for(name)
+    page = TINY[name][1]
+    ref = plain_logits(name, dtype_name)
+    mixed_steps, mixed_pages = cut_mixed(prompts, page)
+    runner = make_runner(tiny_dirs[name], dtype_name, page, num_pages=-(-max(LENGTHS[name]) // page))
+    whole = replay(runner, cut_whole(prompts))
+    for i, p in enumerate(prompts):
+        got = torch.stack([whole[(i, j)] for j in range(len(p))])
+        torch.testing.assert_close(got, ref[i], **TOL[dtype_name], msg=lambda m: f"request {i} (length {len(p)}), whole: {m}")
+    for label, steps, pages in (("tail", cut_tail(prompts), None), ("chunks", cut_chunks(prompts), None),
+                                ("mixed", mixed_steps, mixed_pages)):
+        if pages is not None:
+            runner = make_runner(tiny_dirs[name], dtype_name, page, num_pages=pages)
+        got = replay(runner, steps)
+        assert set(got) == set(whole), label
+        bad = [k for k in sorted(whole) if not torch.equal(got[k], whole[k])]
+        assert not bad, f"{label}: first differing (request, position) {bad[0]} of {len(bad)}; " \
+                        f"max diff {(got[bad[0]] - whole[bad[0]]).abs().max().item():.3e}"
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_page_size_64_and_first_tokens(tiny_dirs, plain_logits, dtype_name):
+    """The default page size, and the first tokens of a sequence one by one from an empty cache."""
+    name = "B"
+    prompts = prompts_for(name)
+    ref = plain_logits(name, dtype_name)
+    runner = make_runner(tiny_dirs[name], dtype_name, 64, num_pages=4)
+    i = 7
+    steps = [([(0, prompts[i][j:j + 1], [0])], []) for j in range(40)]
+    got = replay(runner, steps + [([(0, prompts[i][40:], list(range(len(prompts[i]) - 40)))], [0])])
+    stacked = torch.stack([got[(0, j)] for j in range(len(prompts[i]))])
+    torch.testing.assert_close(stacked, ref[i], **TOL[dtype_name])
+
+
+def test_weights_are_kept_in_their_types(tiny_dirs):
+    from vosti_amd.models import load_model
+    m = load_model(tiny_dirs["A"], "bfloat16")
+    assert m.embedding.weight.dtype == torch.bfloat16 and m.head.weight is m.embedding.weight
+    assert m.layers[0].mixer.w_qkv.dtype == torch.bfloat16
+    m32 = load_model(tiny_dirs["A"], "float32")
+    assert m32.layers[0].mixer.w_qkv.dtype == torch.float32
+
+
+def run_trace(model_dir, dtype_name, out_dir, max_tokens, steps, page_size=None):
+    cmd = [sys.executable, str(ROOT / "bin" / "trace_run"), "--model", str(model_dir), "--dtype", dtype_name, "--out",
+           str(out_dir), "--max-tokens", str(max_tokens)]
+    if page_size:
+        cmd += ["--page-size", str(page_size)]
+    proc = subprocess.Popen(cmd, stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
+    for rec in steps:
+        proc.stdin.write(json.dumps(rec) + "\n")
+        proc.stdin.flush()
+        assert proc.stdout.readline().strip() == f"done {rec['step']}"
+    proc.stdin.close()
+    assert proc.wait(timeout=60) == 0
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_trace_run_program(tiny_dirs, plain_logits, tmp_path, dtype_name):
+    """The command-line tool: two requests interleaved, pages for just these two, then a third
+    request that can only run on pages the first ones gave back."""
+    name = "B"
+    prompts = prompts_for(name)
+    ref = plain_logits(name, dtype_name)
+    a, b, c = 3, 5, 4     # lengths 65, 129, 120
+    vocab = TINY[name][0]["vocab_size"]
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": prompts[a][:40], "want": [0, 39]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": prompts[a][40:], "want": [24]},
+                                {"id": "b", "tokens": prompts[b][:100], "want": []}], "end": ["a"]},
+        {"step": 2, "entries": [{"id": "b", "tokens": prompts[b][100:128], "want": [27]}], "end": []},
+        {"step": 3, "entries": [{"id": "b", "tokens": prompts[b][128:], "want": [0]}], "end": ["b"]},
+        {"step": 4, "entries": [{"id": "c", "tokens": prompts[c], "want": [119]}], "end": ["c"]},
+    ]
+    run_trace(tiny_dirs[name], dtype_name, tmp_path, max_tokens=128 + 192, steps=steps)
+    read = lambda s: torch.from_numpy(np.fromfile(tmp_path / f"{s}.f32", dtype="<f4").reshape(-1, vocab))
+    tol = TOL[dtype_name]
+    torch.testing.assert_close(read(0), ref[a][[0, 39]], **tol)
+    torch.testing.assert_close(read(1), ref[a][[64]], **tol)
+    torch.testing.assert_close(read(2), ref[b][[127]], **tol)
+    torch.testing.assert_close(read(3), ref[b][[128]], **tol)
+    torch.testing.assert_close(read(4), ref[c][[119]], **tol)

@@ -1,0 +1,72 @@
+"""Trace replay: the command-line face of the step function (see bin/trace_run)."""
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+from pathlib import Path
+
+
+def build_parser() -> argparse.ArgumentParser:
+    p = argparse.ArgumentParser(prog="trace_run", description="Replay token traces through the step function and write logits.")
+    p.add_argument("--model", required=True, help="folder with config.json and model.safetensors")
+    p.add_argument("--dtype", required=True, choices=["bfloat16", "float32"],
+                   help="bfloat16: the kernels and precisions of serving; float32: everything in true 32-bit")
+    p.add_argument("--out", required=True, help="folder for <step>.f32 files")
+    p.add_argument("--max-tokens", type=int, required=True,
+                   help="most tokens live requests hold at any time, each request rounded up to a page")
+    p.add_argument("--page-size", type=int, default=64, help="tokens per cache page (a power of two, default 64)")
+    p.add_argument("--max-requests", type=int, default=8, help="most requests alive at a time (state slots)")
+    return p
+
+
+def main(argv: list[str] | None = None) -> int:
+    args = build_parser().parse_args(argv)
+    print("trace_run: loading (native code is compiled at first use)", file=sys.stderr, flush=True)
+    import numpy as np
+    import torch
+
+    if not torch.cuda.is_available():
+        print("trace_run: no GPU visible; this engine has no CPU path", file=sys.stderr)
+        return 2
+    from ..cache import CachePool
+    from ..models import load_model
+    from .step import ModelRunner, StepEntry
+
+    model = load_model(args.model, args.dtype)
+    page = args.page_size
+    num_pages = max(1, -(-args.max_tokens // page))
+    pool = CachePool(model, page_size=page, num_pages=num_pages, num_slots=args.max_requests)
+    runner = ModelRunner(model, pool)
+    out_dir = Path(args.out)
+    out_dir.mkdir(parents=True, exist_ok=True)
+    ids: dict[str, int] = {}     # request names -> numbers; a name may come back after it ended
+    next_id = 0
+    print("trace_run: ready", file=sys.stderr, flush=True)
+    for line in sys.stdin:
+        line = line.strip()
+        if not line:
+            continue
+        rec = json.loads(line)
+        step = rec["step"]
+        entries = []
+        for e in rec.get("entries", []):
+            name = str(e["id"])
+            if name not in ids:
+                ids[name] = next_id
+                next_id += 1
+            entries.append(StepEntry(ids[name], [int(t) for t in e["tokens"]], [int(w) for w in e.get("want", [])]))
+        logits = runner.step(entries)
+        if logits.shape[0] > 0:
+            arr = model.kernels.to_f32(logits).cpu().numpy().astype("<f4", copy=False)
+            arr.tofile(str(out_dir / f"{step}.f32"))
+        else:
+            torch.cuda.synchronize()
+        for name in rec.get("end", []):
+            name = str(name)
+            if name in ids:
+                rid = ids.pop(name)
+                if runner.cache.has_request(rid):
+                    runner.finish(rid)
+        print(f"done {step}", flush=True)
+    return 0

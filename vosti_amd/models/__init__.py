@@ -1,3 +1,3 @@
-from .decoder import DecoderModel, build_model
+from .decoder import DecoderModel, build_model, load_model
 
-__all__ = ["DecoderModel", "build_model"]
+__all__ = ["DecoderModel", "build_model", "load_model"]

@@ -103,3 +103,13 @@ class DecoderModel:
 def build_model(config, dtype) -> DecoderModel:
     """config: an architecture's configuration object (it has ``model_spec()``)."""
     return DecoderModel(config.model_spec(), kernels_for(dtype))
+
+
+def load_model(model_dir, dtype) -> DecoderModel:
+    """A model folder (config.json, safetensors) -> a model with its weights on the GPU.
+    The architecture is chosen by config.json through the registry."""
+    from ..config import load_config
+    from ..weights import load_weights
+    model = build_model(load_config(model_dir), dtype)
+    load_weights(model, model_dir)
+    return model
