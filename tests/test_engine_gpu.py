@@ -1,0 +1,172 @@
+"""The engine end to end: scheduler, step function, sampler, entry points."""
+import json
+import os
+import random
+import subprocess
+import sys
+
+import pytest
+import torch
+
+from conftest import ROOT, TINY
+from plain_qwen3 import PlainQwen3
+
+pytestmark = pytest.mark.gpu
+DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def prompts(name, lengths, seed=3):
+    rng = random.Random(seed)
+    vocab = TINY[name][0]["vocab_size"]
+    return [[rng.randrange(vocab) for _ in range(n)] for n in lengths]
+
+
+def engine(model_dir, dtype, **kw):
+    from vosti_amd.engine import Engine
+    return Engine(model_dir, dtype=dtype, **kw)
+
+
+def check_greedy_against_plain(plain, prompt, out, dtype_name):
+    """Every emitted token is the plain implementation's argmax of the same history; in bfloat16 a
+    token whose plain logit lies within two roundings of the maximum also passes (a near tie)."""
+    ids = list(prompt)
+    for tok in out:
+        row = plain.logits(ids)[-1]
+        if dtype_name == "float32":
+            assert tok == int(torch.argmax(row)), (len(ids), tok)
+        else:
+            assert row[tok] >= row.max() - 2 ** -6 * max(1.0, row.abs().max().item()), (len(ids), tok)
+        ids.append(tok)
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_tiny_a_workload_greedy(tiny_dirs, dtype_name):
+    """Four requests with prompts of 1, 7, 33 and 64 tokens, greedy, 16 new tokens each."""
+    from vosti_amd.sampling import SamplingParams
+    ps = prompts("A", [1, 7, 33, 64])
+    plain = PlainQwen3(tiny_dirs["A"], DTYPES[dtype_name])
+    outs = engine(tiny_dirs["A"], dtype_name, num_pages=24, page_size=16, max_num_seqs=4).generate(ps, SamplingParams(max_tokens=16))
+    assert [len(o) for o in outs] == [16] * 4
+    for p, o in zip(ps, outs):
+        check_greedy_against_plain(plain, p, o, dtype_name)
+    # Alone, with another page size, a small budget and no prefix cache: the same tokens, bit for bit.
+    for i, p in enumerate(ps):
+        alone = engine(tiny_dirs["A"], dtype_name, num_pages=8, page_size=32, max_num_seqs=1, max_num_batched_tokens=16,
+                       enable_prefix_cache=False).generate([p], SamplingParams(max_tokens=16))
+        assert alone[0] == outs[i]
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_tiny_b_workload_temperature_staggered(tiny_dirs, dtype_name):
+    """Six requests, prompts of 2 to 120 tokens, temperature 0.8 with a seed per request, 24 new tokens,
+    staggered arrival; few pages, so that some requests wait and pages are used again."""
+    from vosti_amd.sampling import SamplingParams, uniform_for
+    ps = prompts("B", [2, 120, 31, 64, 9, 77])
+    params = [SamplingParams(max_tokens=24, temperature=0.8, seed=100 + i) for i in range(6)]
+    e = engine(tiny_dirs["B"], dtype_name, num_pages=40, page_size=8, max_num_seqs=3, max_num_batched_tokens=48)
+    outs = e.generate(ps, params, arrival_steps=[0, 0, 2, 4, 8, 12])
+    assert [len(o) for o in outs] == [24] * 6 and e.cache.num_requests() == 0 and e.cache.check() == ""
+    # Each request alone draws the same tokens: nothing depends on the companions or the schedule.
+    for i in (0, 1, 4):
+        alone = engine(tiny_dirs["B"], dtype_name, num_pages=32, page_size=8, max_num_seqs=1).generate([ps[i]], params[i])
+        assert alone[0] == outs[i], i
+    # Against the plain implementation: the drawn token's interval of the plain CDF holds the same uniform number.
+    plain = PlainQwen3(tiny_dirs["B"], DTYPES[dtype_name])
+    slack = 1e-4 if dtype_name == "float32" else 2e-2
+    for i in (0, 2):
+        ids = list(ps[i])
+        for j, tok in enumerate(outs[i]):
+            p = torch.softmax(plain.logits(ids)[-1].double() / 0.8, 0)
+            cdf = torch.cumsum(p, 0)
+            u = uniform_for(params[i].seed, j)
+            lo = cdf[tok - 1].item() if tok else 0.0
+            assert lo - slack <= u <= cdf[tok].item() + slack, (i, j)
+            ids.append(tok)
+    # Different seeds give different continuations; temperature 0 in the same batch stays greedy.
+    assert outs[0] != engine(tiny_dirs["B"], dtype_name, num_pages=32, page_size=8).generate([ps[0]], SamplingParams(max_tokens=24, temperature=0.8, seed=7))[0]
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_prefix_cache_hit_equals_cold_run(tiny_dirs, dtype_name):
+    from vosti_amd.sampling import SamplingParams
+    shared = prompts("B", [70], seed=9)[0]
+    a, b = shared + [1, 2, 3], shared + [4]
+    sp = SamplingParams(max_tokens=8)
+    cold = engine(tiny_dirs["B"], dtype_name, num_pages=32, page_size=8, enable_prefix_cache=False)
+    want_b = cold.generate([b], sp)[0]
+    warm = engine(tiny_dirs["B"], dtype_name, num_pages=32, page_size=8, enable_prefix_cache=True)
+    warm.generate([a], sp)
+    assert warm.generate([b], sp)[0] == want_b and warm.cache.prefix_hits() == 8      # 64 of 70 shared tokens
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_long_decoding_equals_whole_prompt(tiny_dirs, dtype_name):
+    """200 decoded tokens from a short prompt; then the whole sequence in one step: the logits at every
+    decoded position are the same bits, so every emitted token is the whole-prompt argmax."""
+    from vosti_amd.engine import StepEntry
+    from vosti_amd.sampling import SamplingParams
+    p = prompts("B", [5], seed=4)[0]
+    e = engine(tiny_dirs["B"], dtype_name, num_pages=40, page_size=8, max_num_seqs=2)
+    out = e.generate([p], SamplingParams(max_tokens=200))[0]
+    seq = p + out
+    logits = e.runner.step([StepEntry(12345, seq[:-1], list(range(len(p) - 1, len(seq) - 1)))])
+    e.runner.finish(12345)
+    assert e.kernels.sample(logits).cpu().tolist() == out
+
+
+def test_pages_run_out_through_the_engine(tiny_dirs):
+    """So few pages that requests are preempted and recomputed: the tokens are still those of a roomy run."""
+    from vosti_amd.cache import OutOfPages
+    from vosti_amd.sampling import SamplingParams
+    ps = prompts("A", [20, 25, 30, 18], seed=6)
+    sp = SamplingParams(max_tokens=40)
+    roomy = engine(tiny_dirs["A"], "float32", num_pages=64, page_size=8, max_num_seqs=4).generate(ps, sp)
+    tight_engine = engine(tiny_dirs["A"], "float32", num_pages=20, page_size=8, max_num_seqs=4)
+    assert tight_engine.generate(ps, sp) == roomy and tight_engine.scheduler.preemptions() > 0
+    with pytest.raises(OutOfPages):
+        engine(tiny_dirs["A"], "float32", num_pages=2, page_size=8).generate([ps[0]], sp)
+
+
+def test_refusals(tiny_dirs):
+    from vosti_amd.sampling import SamplingParams
+    e = engine(tiny_dirs["A"], "float32", num_pages=8, page_size=16)
+    with pytest.raises(ValueError, match="EmptyPrompt"):
+        e.add_request([])
+    with pytest.raises(ValueError, match="outside"):
+        e.add_request([256])
+    with pytest.raises(ValueError, match="HistoryCapacityOverflow"):
+        e.add_request([1] * 100, SamplingParams(max_tokens=29))      # 128 positions
+    with pytest.raises(ValueError):
+        engine(tiny_dirs["A"], "float32", num_pages=8, page_size=12)      # not a power of two
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_command_line(tiny_dirs, tmp_path, dtype_name):
+    """The launcher with the reference's environment variables; output as the reference prints it."""
+    p = prompts("A", [9], seed=8)[0]
+    env = dict(os.environ, MODEL_PATH=str(tiny_dirs["A"]), VOSTI_PROMPT_IDS=",".join(map(str, p)), VOSTI_MAX_TOKENS="5",
+               VOSTI_NUM_BLOCKS="4", VOSTI_DTYPE=dtype_name, VOSTI_OUTPUT_TOKENS=str(tmp_path / "out.tsv"),
+               VOSTI_ENGINE_STEP_TRACE=str(tmp_path / "trace.jsonl"), PYTHONPATH=str(ROOT))
+    r = subprocess.run([sys.executable, "-m", "vosti_amd.launch", "--kind", "engine", "--family", "qwen3"], env=env,
+                       capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0, r.stderr[-2000:]
+    line = [l for l in r.stdout.splitlines() if l.startswith("MODEL_OUTPUT_TOKEN_IDS=")][0]
+    out = json.loads(line.split("=", 1)[1])
+    check_greedy_against_plain(PlainQwen3(tiny_dirs["A"], DTYPES[dtype_name]), p, out, dtype_name)
+    assert (tmp_path / "out.tsv").read_text() == "0\t" + ",".join(map(str, out)) + "\n"
+    steps = [json.loads(l) for l in (tmp_path / "trace.jsonl").read_text().splitlines()]
+    assert len(steps) == 5 and steps[0]["arrived"] == [0] and steps[-1]["emitted"] == {"0": out[-1]}
+    # Prepared requests: MAX_TOKENS <TAB> IDS [<TAB> ARRIVAL_STEP], one BENCH line.
+    (tmp_path / "reqs.tsv").write_text("# two requests\n3\t1,2,3\n4\t7,8\t2\n")
+    env2 = dict(env, VOSTI_BENCH_INPUT=str(tmp_path / "reqs.tsv"))
+    r = subprocess.run([sys.executable, "-m", "vosti_amd.launch", "--kind", "engine", "--family", "qwen3", "--",
+                        "--output-tokens", str(tmp_path / "o2.tsv")], env=env2, capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert "BENCH batch=2 prompt_tokens=5 output_tokens=7" in r.stdout
+    assert [len(l.split("\t")[1].split(",")) for l in (tmp_path / "o2.tsv").read_text().splitlines()] == [3, 4]
+
+
+def test_smoke_entry():
+    sys.path.insert(0, str(ROOT))
+    import __graft_entry__
+    __graft_entry__.smoke()

@@ -1,0 +1,181 @@
+"""Command line of the engine, in the manner of the reference's launcher.
+
+    python -m vosti_amd.launch --kind engine --family qwen3 [-- options]
+    python -m vosti_amd.launch --kind random-model --family qwen3 -- --config CONFIG.json --seed N --out DIR
+
+The reference starts its engine example through ``scripts/launch.py --kind engine
+--family qwen3`` (scripts/launch.py:17-55) and configures it by environment
+variables (examples/support/engine_setup.rs:57-69, 110-118;
+examples/support/engine_serving.rs:75-231).  The same variables mean the same
+here; each also has a command-line option, which wins:
+
+    MODEL_PATH                 --model-path          model folder (required)
+    CUDA_DEVICE                --device              only cuda:0 exists here
+    VOSTI_PROMPT_IDS           --prompt-ids          comma-separated token ids (default "9707")
+    VOSTI_MAX_TOKENS           --max-tokens          new tokens (default 8)
+    VOSTI_IGNORE_EOS           --ignore-eos          presence: do not stop on end tokens
+    VOSTI_NUM_BLOCKS           --num-blocks          cache pages (default 32)
+    VOSTI_MAX_SEQS             --max-seqs            rows per step (default: the batch size)
+    VOSTI_MAX_BATCHED_TOKENS   --max-batched-tokens  tokens per step (default 4096)
+    VOSTI_OUTPUT_TOKENS        --output-tokens       write "index<TAB>ids" lines to this file
+    VOSTI_BENCH_INPUT          --bench-input         TSV of MAX_TOKENS<TAB>IDS[<TAB>ARRIVAL_STEP] requests
+    VOSTI_ENGINE_STEP_TRACE    --step-trace          append one JSON line per step to this file
+
+Options without a counterpart in the reference: VOSTI_DTYPE / --dtype (bfloat16,
+float32), VOSTI_TEMPERATURE / --temperature, VOSTI_SEED / --seed,
+VOSTI_PAGE_SIZE / --page-size, VOSTI_PREFIX_CACHE / --prefix-cache (0, 1).
+End tokens come from generation_config.json's ``eos_token_id`` (one to three
+ids: python/vosti_kernels/serving_workload.py:78-108); without that file there
+are none.  It prints ``MODEL_OUTPUT_TOKEN_IDS=[...]`` like the reference, or a
+``BENCH batch=... tok_s=...`` line for prepared requests.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+FAMILIES = {"qwen3": "Qwen3ForCausalLM"}
+
+
+def _env(name: str, default=None):
+    v = os.environ.get(name)
+    return default if v is None or v == "" else v
+
+
+def engine_parser() -> argparse.ArgumentParser:
+    p = argparse.ArgumentParser(prog="vosti_amd.launch --kind engine", description="Generate tokens for prompts given as token ids.")
+    p.add_argument("--model-path", default=_env("MODEL_PATH"))
+    p.add_argument("--device", default=_env("CUDA_DEVICE", "cuda:0"))
+    p.add_argument("--prompt-ids", default=_env("VOSTI_PROMPT_IDS", "9707"))
+    p.add_argument("--max-tokens", type=int, default=int(_env("VOSTI_MAX_TOKENS", 8)))
+    p.add_argument("--ignore-eos", action="store_true", default="VOSTI_IGNORE_EOS" in os.environ)
+    p.add_argument("--num-blocks", type=int, default=int(_env("VOSTI_NUM_BLOCKS", 32)))
+    p.add_argument("--max-seqs", type=int, default=int(_env("VOSTI_MAX_SEQS", 0)))
+    p.add_argument("--max-batched-tokens", type=int, default=int(_env("VOSTI_MAX_BATCHED_TOKENS", 4096)))
+    p.add_argument("--output-tokens", default=_env("VOSTI_OUTPUT_TOKENS"))
+    p.add_argument("--bench-input", default=_env("VOSTI_BENCH_INPUT"))
+    p.add_argument("--step-trace", default=_env("VOSTI_ENGINE_STEP_TRACE"))
+    p.add_argument("--dtype", default=_env("VOSTI_DTYPE", "bfloat16"), choices=["bfloat16", "float32"])
+    p.add_argument("--temperature", type=float, default=float(_env("VOSTI_TEMPERATURE", 0.0)))
+    p.add_argument("--seed", type=int, default=int(_env("VOSTI_SEED", 0)))
+    p.add_argument("--page-size", type=int, default=int(_env("VOSTI_PAGE_SIZE", 64)))
+    p.add_argument("--prefix-cache", type=int, default=int(_env("VOSTI_PREFIX_CACHE", 1)), choices=[0, 1])
+    return p
+
+
+def parse_ids(text: str) -> list[int]:
+    try:
+        ids = [int(x) for x in text.replace(" ", "").split(",") if x != ""]
+    except ValueError:
+        raise SystemExit(f"prompt ids must be comma-separated integers, got {text!r}") from None
+    if not ids:
+        raise SystemExit("the prompt is empty")
+    return ids
+
+
+def parse_prepared(path: str) -> list[tuple[int, list[int], int]]:
+    """MAX_TOKENS<TAB>IDS[<TAB>ARRIVAL_STEP] per line; '#' starts a comment
+    (examples/support/engine_benchmark.rs:79-165)."""
+    out = []
+    for n, line in enumerate(Path(path).read_text().splitlines(), 1):
+        if not line.strip() or line.lstrip().startswith("#"):
+            continue
+        f = line.split("\t")
+        if len(f) not in (2, 3):
+            raise SystemExit(f"{path}:{n}: expected MAX_TOKENS<TAB>IDS[<TAB>ARRIVAL_STEP]")
+        out.append((int(f[0]), parse_ids(f[1]), int(f[2]) if len(f) == 3 else 0))
+    if not out:
+        raise SystemExit(f"{path} holds no requests")
+    return out
+
+
+def eos_ids(model_path: str) -> tuple[int, ...]:
+    path = Path(model_path) / "generation_config.json"
+    if not path.is_file():
+        return ()
+    v = json.loads(path.read_text()).get("eos_token_id")
+    if v is None:
+        return ()
+    ids = [v] if isinstance(v, int) else list(v)
+    if not 1 <= len(ids) <= 3:
+        raise SystemExit("generation_config.json: 'eos_token_id' must hold one to three ids")
+    return tuple(int(i) for i in ids)
+
+
+def run_engine(argv: list[str], family: str) -> int:
+    args = engine_parser().parse_args(argv)
+    if not args.model_path:
+        raise SystemExit("MODEL_PATH (or --model-path) is required")
+    if args.device not in ("cuda:0", "cuda"):
+        raise SystemExit(f"device {args.device!r}: this engine runs on cuda:0 only")
+    from .config import load_config
+    cfg = load_config(args.model_path)
+    if cfg.architecture != FAMILIES[family]:
+        raise SystemExit(f"{args.model_path} holds a {cfg.architecture}, not a {family} model")
+    from .engine import Engine
+    from .sampling import SamplingParams
+    if args.bench_input:
+        requests = parse_prepared(args.bench_input)
+    else:
+        requests = [(args.max_tokens, parse_ids(args.prompt_ids), 0)]
+    eos = eos_ids(args.model_path)
+    engine = Engine(args.model_path, dtype=args.dtype, num_pages=args.num_blocks, page_size=args.page_size,
+                    max_num_seqs=args.max_seqs or len(requests), max_num_batched_tokens=args.max_batched_tokens,
+                    enable_prefix_cache=bool(args.prefix_cache))
+    params = [SamplingParams(max_tokens=m, temperature=args.temperature, seed=args.seed + i, eos_token_ids=eos,
+                             ignore_eos=args.ignore_eos) for i, (m, _, _) in enumerate(requests)]
+    trace = open(args.step_trace, "a") if args.step_trace else None
+    import torch
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    outputs = engine.generate([ids for _, ids, _ in requests], params, [a for _, _, a in requests], trace=trace)
+    wall = time.perf_counter() - t0
+    if trace:
+        trace.close()
+    if args.output_tokens:
+        Path(args.output_tokens).write_text("".join(f"{i}\t{','.join(map(str, o))}\n" for i, o in enumerate(outputs)))
+    if args.bench_input:
+        n_out = sum(len(o) for o in outputs)
+        print(f"BENCH batch={len(requests)} prompt_tokens={sum(len(i) for _, i, _ in requests)} output_tokens={n_out} "
+              f"wall_s={wall:.9f} tok_s={n_out / wall:.6f}")
+        print("CACHE_STATS " + json.dumps({"admitted_requests": len(requests), "reused_prefix_blocks": engine.cache.prefix_hits(),
+                                           "preemptions": engine.scheduler.preemptions()}, separators=(",", ":")))
+    else:
+        print(f"MODEL_OUTPUT_TOKEN_IDS={outputs[0]}")
+    return 0
+
+
+def run_random_model(argv: list[str], family: str) -> int:
+    p = argparse.ArgumentParser(prog="vosti_amd.launch --kind random-model",
+                                description="Write a model folder (config.json, model.safetensors) with random weights.")
+    p.add_argument("--config", required=True, help="a config.json of the architecture")
+    p.add_argument("--seed", type=int, default=0)
+    p.add_argument("--out", required=True)
+    p.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    args = p.parse_args(argv)
+    import torch
+    from .config import config_from_dict
+    from .weights import write_random_model
+    raw = json.loads(Path(args.config).read_text())
+    raw.setdefault("architectures", [FAMILIES[family]])
+    out = write_random_model(config_from_dict(raw), args.seed, args.out, getattr(torch, args.dtype))
+    print(f"wrote {out}")
+    return 0
+
+
+def main(argv: list[str] | None = None) -> int:
+    p = argparse.ArgumentParser(description="Launch the engine or write a random-weights model folder.")
+    p.add_argument("--kind", required=True, choices=("engine", "random-model"))
+    p.add_argument("--family", required=True, choices=sorted(FAMILIES))
+    p.add_argument("args", nargs=argparse.REMAINDER, help="options of the chosen kind, after --")
+    ns = p.parse_args(argv)
+    rest = ns.args[1:] if ns.args[:1] == ["--"] else ns.args
+    return run_engine(rest, ns.family) if ns.kind == "engine" else run_random_model(rest, ns.family)
+
+
+if __name__ == "__main__":
+    sys.exit(main())
