@@ -28,7 +28,8 @@ def rand(shape, dtype, seed, scale=1.0):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,N,K", [(1, 64, 64), (5, 503, 96), (17, 224, 96), (64, 256, 224), (16, 48, 520),
-                                   (65, 130, 520), (130, 96, 1032), (300, 520, 2056), (8, 40, 4104)])
+                                   (65, 130, 520), (130, 96, 1032), (300, 520, 2056), (8, 40, 4104),
+                                   (8, 4100, 1024), (3, 72, 512), (33, 200, 1536), (64, 4096, 4608), (17, 90, 5120)])
 def test_gemm(dtype, M, N, K):
     k = kern(dtype)
     a, w = rand((M, K), dtype, 1), rand((N, K), dtype, 2, 0.1)
@@ -281,12 +282,9 @@ def run_attention(k, q_list, kk, vv, P, dtype, window=0, poison=None, decode_spl
         k.paged_attention(*args, torch.tensor(pre, dtype=torch.int32).cuda(), mode=0, **kw)
     if dec:
         items = torch.tensor(dec, dtype=torch.int32).cuda()
-        if decode_split:
-            nseg = -(-int(k_len.max()) // 256) + 1
-            scratch = torch.full((k.attn_scratch_floats(q.shape[0], q.shape[1], d, nseg),), float("nan"), device="cuda")
-            k.paged_attention(*args, items, mode=1, split=True, nseg=nseg, scratch=scratch, **kw)
-        else:
-            k.paged_attention(*args, items, mode=1, **kw)
+        nseg = -(-int(k_len.max()) // 256) + (1 if decode_split else 0)    # more segments than needed are harmless
+        scratch = torch.full((k.attn_scratch_floats(q.shape[0], q.shape[1], d, nseg),), float("nan"), device="cuda")
+        k.paged_attention(*args, items, mode=1, nseg=nseg, scratch=scratch, **kw)
     return out.cpu()
 
 
@@ -309,7 +307,7 @@ def test_attention_against_plain(dtype, nq, nkv, d, P):
         ref = plain.attention(q, kx, vx, d ** -0.5, dtype)
         torch.testing.assert_close(got[off:off + q.shape[0]].float(), ref, **tol(dtype))
         off += q.shape[0]
-    # Poison changes nothing bitwise; the split decode path gives the same bits as the fused one.
+    # Poison changes nothing bitwise, nor does another page order or a wider segment grid.
     clean = run_attention(k, q_list, kk, vv, P, dtype, poison=None, decode_split=True, seed=5)
     assert torch.equal(clean, got)
 
@@ -378,4 +376,4 @@ def test_attention_refuses_bad_sizes():
     i32 = lambda *v: torch.tensor(v, dtype=torch.int32, device="cuda")
     with pytest.raises(KernelError, match="head size"):
         k.paged_attention(q, kc, vc, i32(0, 1).view(1, 2), i32(0, 1), i32(1), i32(0, 0).view(1, 2), mode=1, scale=1.0,
-                          max_k_len=1)
+                          max_k_len=1, nseg=1, scratch=torch.zeros(64, device="cuda"))

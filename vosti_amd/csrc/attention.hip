@@ -10,17 +10,21 @@
 // tile in which a row sees no key leaves that row's state untouched; out =
 // acc / l (0 if l == 0).
 //
-// Reduction order (a function of absolute key positions only, so that any cut
-// of a sequence into steps, and any split of the keys over workgroups, gives
-// the same bits):
-//   keys are grouped in tiles of 64 (positions 64t .. 64t+63) and tiles in
-//   segments of 4 (256 keys).  Within a segment the state (m, l, acc) starts
-//   at (-inf, 0, 0) and is updated tile by tile, ascending, by online softmax.
-//   Segment results are merged into the total, ascending:
-//     M' = max(M, m); ACC' = ACC * 2^(M - M') + acc * 2^(m - M'); L' likewise.
-//   A workgroup either walks all segments of its rows and merges in registers
-//   (prompt portions), or takes one segment and leaves (m, l, acc) in a
-//   scratch buffer that attn_combine merges with the same formula (decode).
+// Reduction order.  It is a function of absolute key positions only, so that
+// any cut of a sequence into steps, and any split of the keys over waves and
+// workgroups, gives the same bits:
+//   tile     64 keys, positions 64t .. 64t+63.  Each tile is reduced on its
+//            own: m = max of the visible scores, p = 2^(s - m), l = sum p,
+//            acc = P V accumulated from zero.  A tile without a visible key is
+//            empty (m = -inf).
+//   segment  4 tiles (256 keys).  Its non-empty tiles are folded, ascending,
+//            into a state that starts empty:
+//              M' = max(M, m); ACC' = ACC * 2^(M - M') + acc * 2^(m - M'); L' likewise.
+//   total    the non-empty segments are folded, ascending, the same way.
+// The prompt kernel folds in registers as it walks the tiles.  The decode
+// kernel gives every tile of a segment to a wave of its own, folds the four in
+// LDS and leaves the segment's (m, l, acc) in a scratch buffer that
+// attn_combine folds; the arithmetic is the same sequence of fp32 operations.
 //
 // Cache layout: keys [pages, nkv, page, d]; values transposed [pages, nkv, d, page],
 // so that both MFMA operands of both products are 16-byte loads from global
@@ -44,225 +48,239 @@ struct AttnArgs {
   const int32_t* cu_q;    // [S + 1]
   const int32_t* k_len;   // [S]
   const int32_t* items;   // [n_items, 2]: (sequence, first row of the item within the step's rows of it)
-  float* part_ml;         // split: [T * nq * nseg, 2]
-  float* part_acc;        // split: [T * nq * nseg, d]
+  float* part_ml;         // decode: [T * nq * nseg, 2]
+  float* part_acc;        // decode: [T * nq * nseg, d]
   int bt_stride, nq, nkv, d, P, window, nseg;
   float scale_log2;
 };
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-// MODE 0: the 16 rows of a wave are 16 consecutive tokens of one q head.
-// MODE 1: the 16 rows are up to 16 q heads of one kv head, for one token.
-template <int DPAD, int MODE, bool SPLIT>
-__global__ __launch_bounds__(64) void attn_kernel(AttnArgs a) {
-  constexpr int NDT = DPAD / 16;          // output d tiles
-  constexpr int NQS = DPAD / VK_SLAB;     // slabs along d
-  const int lane = threadIdx.x, r16 = lane & 15, g = lane >> 4;
+// What a wave needs to know about its 16 rows and its sequence's pages.
+struct RowCtx {
+  const int32_t* bt;
+  const elem_t* kbase;     // + kv head offset
+  const elem_t* vbase;
+  int64_t page_stride;
+  int k_len, d, P, r16, g;
+  int lo, pos;             // this lane's row sees keys lo..pos
+  int wave_lo;             // smallest key any row of the wave sees
+  bool row_ok;
+  float scale_log2;
+};
+
+// One tile, reduced on its own: m, l and acc[NDT] of this lane's row.
+template <int NDT, int NQS>
+__device__ __forceinline__ void tile_partial(const RowCtx& c, const frag_t (&qf)[NQS], int kb, float& m_t, float& l_t,
+                                             f32x4 (&acc)[NDT]) {
+  const int d = c.d, P = c.P, r16 = c.r16, g = c.g;
+  // ---- scores S^T[key, row] = K Q^T ----
+  float sc[S_PER_LANE];
+#pragma unroll
+  for (int ks = 0; ks < KEY_SLABS; ++ks) {
+#ifdef VK_BF16
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      // MFMA row m of this sub-tile is key  slab + 8*(m/4) + 4*u + m%4, so that
+      // lane group g ends up with the 8 consecutive keys slab + 8g .. 8g+7.
+      const int key = kb + ks * VK_SLAB + 8 * (r16 >> 2) + 4 * u + (r16 & 3);
+#else
+    {
+      const int u = 0;
+      const int key = kb + ks * VK_SLAB + r16;
+#endif
+      const bool kok = key < c.k_len;
+      const int kk = kok ? key : 0;
+      const int page = c.bt[kk / P];
+      const elem_t* krow = c.kbase + page * c.page_stride + (int64_t)(kk % P) * d;
+      f32x4 s4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < NQS; ++s) {
+        if (s * VK_SLAB < d) {
+          const int col = s * VK_SLAB + g * VK_VEC;
+          const frag_t kf = load_frag(krow + col, kok && col < d);
+          s4 = mma_slab(kf, qf[s], s4);
+        }
+      }
+      sc[ks * VK_VEC + 4 * u + 0] = s4.x;
+      sc[ks * VK_VEC + 4 * u + 1] = s4.y;
+      sc[ks * VK_VEC + 4 * u + 2] = s4.z;
+      sc[ks * VK_VEC + 4 * u + 3] = s4.w;
+    }
+  }
+  // ---- value fragments: requested before the softmax arithmetic needs them ----
+  // Keys outside [wave_lo, k_len) may lie in pages this sequence does not own
+  // (never written, or given back once the window passed them): their values
+  // are replaced by zero so that stale NaN or Inf cannot reach the sum.
+  const bool edge = kb + TILE_KEYS > c.k_len || kb < c.wave_lo;
+  frag_t vf[NDT][KEY_SLABS];
+#pragma unroll
+  for (int dt = 0; dt < NDT; ++dt) {
+    if (dt * 16 < d) {
+#pragma unroll
+      for (int ks = 0; ks < KEY_SLABS; ++ks) {
+        const int k0 = kb + ks * VK_SLAB + g * VK_VEC;
+        const bool vok = k0 < c.k_len;
+        const int kk = vok ? k0 : 0;
+        const int page = c.bt[kk / P];
+        const elem_t* vrow = c.vbase + page * c.page_stride + (int64_t)(dt * 16 + r16) * P + (kk % P);
+        vf[dt][ks] = load_frag(vrow, vok);
+        if (edge) {
+#pragma unroll
+          for (int j = 0; j < VK_VEC; ++j)
+            if (k0 + j >= c.k_len || k0 + j < c.wave_lo) vf[dt][ks][j] = (elem_t)0.f;
+        }
+      }
+    }
+  }
+  // ---- mask, maximum, probabilities ----
+  bool vis[S_PER_LANE];
+  float tmax = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < S_PER_LANE; ++i) {
+    const int key = kb + (i / VK_VEC) * VK_SLAB + g * VK_VEC + (i % VK_VEC);
+    vis[i] = c.row_ok && key >= c.lo && key <= c.pos;
+    sc[i] = sc[i] * c.scale_log2;
+    tmax = fmaxf(tmax, vis[i] ? sc[i] : -INFINITY);
+  }
+  tmax = fmaxf(tmax, __shfl_xor(tmax, 16, VK_WAVE));
+  tmax = fmaxf(tmax, __shfl_xor(tmax, 32, VK_WAVE));
+  float psum = 0.f;
+  float pr[S_PER_LANE];
+#pragma unroll
+  for (int i = 0; i < S_PER_LANE; ++i) {
+    pr[i] = vis[i] ? fast_exp2(sc[i] - tmax) : 0.f;
+    psum = psum + pr[i];
+  }
+  psum = psum + __shfl_xor(psum, 16, VK_WAVE);
+  psum = psum + __shfl_xor(psum, 32, VK_WAVE);
+  m_t = tmax;
+  l_t = psum;
+  // ---- acc = V^T P^T from zero; P rounded to the element type ----
+  frag_t pf[KEY_SLABS];
+#pragma unroll
+  for (int ks = 0; ks < KEY_SLABS; ++ks) {
+#ifdef VK_BF16
+#pragma unroll
+    for (int j = 0; j < 8; ++j) pf[ks][j] = (__bf16)pr[ks * 8 + j];
+#else
+    pf[ks] = f32x4{pr[ks * 4 + 0], pr[ks * 4 + 1], pr[ks * 4 + 2], pr[ks * 4 + 3]};
+#endif
+  }
+#pragma unroll
+  for (int dt = 0; dt < NDT; ++dt) {
+    acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (dt * 16 < d) {
+#pragma unroll
+      for (int ks = 0; ks < KEY_SLABS; ++ks) acc[dt] = mma_slab(vf[dt][ks], pf[ks], acc[dt]);
+    }
+  }
+}
+
+// state (M, L, ACC) <- fold of a non-empty partial (m, l, acc).
+__device__ __forceinline__ void fold_scales(float M, float m, float& Mn, float& ca, float& cb) {
+  Mn = fmaxf(M, m);
+  ca = fast_exp2(M - Mn);
+  cb = fast_exp2(m - Mn);
+}
+__device__ __forceinline__ float fold1(float A, float a, float ca, float cb) { return A * ca + a * cb; }
+
+template <int NDT>
+__device__ __forceinline__ void fold(float& M, float& L, f32x4 (&ACC)[NDT], float m, float l, const f32x4 (&acc)[NDT]) {
+  if (!(m > -INFINITY)) return;
+  float Mn, ca, cb;
+  fold_scales(M, m, Mn, ca, cb);
+#pragma unroll
+  for (int dt = 0; dt < NDT; ++dt) {
+    ACC[dt].x = fold1(ACC[dt].x, acc[dt].x, ca, cb);
+    ACC[dt].y = fold1(ACC[dt].y, acc[dt].y, ca, cb);
+    ACC[dt].z = fold1(ACC[dt].z, acc[dt].z, ca, cb);
+    ACC[dt].w = fold1(ACC[dt].w, acc[dt].w, ca, cb);
+  }
+  L = fold1(L, l, ca, cb);
+  M = Mn;
+}
+
+template <int NQS>
+__device__ __forceinline__ void load_q(const AttnArgs& a, int tok, int head, bool row_ok, int g, frag_t (&qf)[NQS]) {
+  const elem_t* qrow = a.q + ((int64_t)(row_ok ? tok : 0) * a.nq + (row_ok ? head : 0)) * a.d;
+#pragma unroll
+  for (int s = 0; s < NQS; ++s) {
+    const int col = s * VK_SLAB + g * VK_VEC;
+    qf[s] = load_frag(qrow + col, row_ok && col < a.d);
+  }
+}
+
+__device__ __forceinline__ void init_ctx(RowCtx& c, const AttnArgs& a, int seq, int kvh, int k_len) {
+  const int64_t page_elems = (int64_t)a.P * a.d;
+  c.bt = a.block_table + (int64_t)seq * a.bt_stride;
+  c.kbase = a.kc + (int64_t)kvh * page_elems;
+  c.vbase = a.vc + (int64_t)kvh * page_elems;
+  c.page_stride = (int64_t)a.nkv * page_elems;
+  c.k_len = k_len;
+  c.d = a.d;
+  c.P = a.P;
+  c.scale_log2 = a.scale_log2;
+}
+
+// Prompt portions: an item is up to 16 consecutive rows of one sequence.  A
+// workgroup has one wave per q head of a kv head (up to 4), so that the waves
+// of a group read the same keys and values at about the same time.
+template <int DPAD>
+__global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a, int heads_per_wg) {
+  constexpr int NDT = DPAD / 16, NQS = DPAD / VK_SLAB;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int G = a.nq / a.nkv;
+  const int groups_per_kv = (G + heads_per_wg - 1) / heads_per_wg;
+  const int kvh = blockIdx.y / groups_per_kv;
+  const int hg = (blockIdx.y - kvh * groups_per_kv) * heads_per_wg + wave;
+  if (hg >= G) return;
+  const int head = kvh * G + hg;
   const int seq = a.items[2 * blockIdx.x], q_off = a.items[2 * blockIdx.x + 1];
   const int q_begin = a.cu_q[seq], q_len = a.cu_q[seq + 1] - q_begin;
   const int k_len = a.k_len[seq];
-  const int G = a.nq / a.nkv;
-  const int d = a.d, P = a.P;
-
-  int tok, head, kvh, pos, nvalid;
-  if (MODE == 0) {
-    head = blockIdx.y;
-    kvh = head / G;
-    nvalid = min(16, q_len - q_off);
-    tok = q_begin + q_off + r16;
-    pos = k_len - q_len + q_off + r16;
-  } else {
-    const int HT = (G + 15) >> 4;
-    kvh = blockIdx.y / HT;
-    const int ht = blockIdx.y - kvh * HT;
-    nvalid = min(16, G - ht * 16);
-    head = kvh * G + ht * 16 + r16;
-    tok = q_begin + q_off;
-    pos = k_len - q_len + q_off;
-  }
-  const bool row_ok = r16 < nvalid;
-  const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
-  // Key range that any row of this wave sees.
+  RowCtx c;
+  init_ctx(c, a, seq, kvh, k_len);
+  c.r16 = lane & 15;
+  c.g = lane >> 4;
+  const int nvalid = min(16, q_len - q_off);
+  c.row_ok = c.r16 < nvalid;
+  const int tok = q_begin + q_off + c.r16;
   const int pos0 = k_len - q_len + q_off;
-  const int wave_hi = MODE == 0 ? pos0 + nvalid - 1 : pos0;
-  const int wave_lo = a.window > 0 ? max(0, pos0 - a.window + 1) : 0;
-  const int tile_lo = wave_lo / TILE_KEYS, tile_hi = wave_hi / TILE_KEYS;
-  int seg_begin = tile_lo / SEG_TILES, seg_end = tile_hi / SEG_TILES + 1;
-  if (SPLIT) {
-    const int seg = blockIdx.z;
-    if (seg < seg_begin || seg >= seg_end) return;
-    seg_begin = seg;
-    seg_end = seg + 1;
-  }
+  c.pos = pos0 + c.r16;
+  c.lo = a.window > 0 ? max(0, c.pos - a.window + 1) : 0;
+  c.wave_lo = a.window > 0 ? max(0, pos0 - a.window + 1) : 0;
+  const int tile_lo = c.wave_lo / TILE_KEYS, tile_hi = (pos0 + nvalid - 1) / TILE_KEYS;
 
-  const int32_t* bt = a.block_table + (int64_t)seq * a.bt_stride;
-  const int64_t page_elems = (int64_t)P * d;       // elements of one (page, kv head)
-  const elem_t* kbase = a.kc + (int64_t)kvh * page_elems;
-  const elem_t* vbase = a.vc + (int64_t)kvh * page_elems;
-  const int64_t page_stride = (int64_t)a.nkv * page_elems;
-
-  // Query fragments: second MFMA operand, lane (row r16, column group g).
   frag_t qf[NQS];
-  {
-    const elem_t* qrow = a.q + ((int64_t)tok * a.nq + head) * d;
-#pragma unroll
-    for (int s = 0; s < NQS; ++s) {
-      const int c = s * VK_SLAB + g * VK_VEC;
-      qf[s] = load_frag(qrow + (row_ok ? c : 0), row_ok && c < d);
-    }
-  }
+  load_q<NQS>(a, tok, head, c.row_ok, c.g, qf);
 
-  float M_tot = -INFINITY, L_tot = 0.f;
+  float M = -INFINITY, L = 0.f;
   f32x4 ACC[NDT];
 #pragma unroll
   for (int dt = 0; dt < NDT; ++dt) ACC[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-  for (int seg = seg_begin; seg < seg_end; ++seg) {
-    float m_run = -INFINITY, l_run = 0.f;
-    f32x4 acc[NDT];
+  for (int seg = tile_lo / SEG_TILES; seg <= tile_hi / SEG_TILES; ++seg) {
+    float Ms = -INFINITY, Ls = 0.f;
+    f32x4 As[NDT];
 #pragma unroll
-    for (int dt = 0; dt < NDT; ++dt) acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-    const int t_begin = max(tile_lo, seg * SEG_TILES), t_end = min(tile_hi, seg * SEG_TILES + SEG_TILES - 1);
-    for (int t = t_begin; t <= t_end; ++t) {
-      const int kb = t * TILE_KEYS;
-      // ---- scores S^T[key, row] = K Q^T ----
-      float sc[S_PER_LANE];
-#pragma unroll
-      for (int ks = 0; ks < KEY_SLABS; ++ks) {
-#ifdef VK_BF16
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-          // MFMA row m of this sub-tile is key  slab + 8*(m/4) + 4*u + m%4, so that
-          // lane group g ends up with the 8 consecutive keys slab + 8g .. 8g+7.
-          const int key = kb + ks * VK_SLAB + 8 * (r16 >> 2) + 4 * u + (r16 & 3);
-#else
-        {
-          const int u = 0;
-          const int key = kb + ks * VK_SLAB + r16;
-#endif
-          const bool kok = key < k_len;
-          const int kk = kok ? key : 0;
-          const int page = bt[kk / P];
-          const elem_t* krow = kbase + page * page_stride + (int64_t)(kk % P) * d;
-          f32x4 s4 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-          for (int s = 0; s < NQS; ++s) {
-            if (s * VK_SLAB < d) {
-              const int c = s * VK_SLAB + g * VK_VEC;
-              const frag_t kf = load_frag(krow + c, kok && c < d);
-              s4 = mma_slab(kf, qf[s], s4);
-            }
-          }
-          sc[ks * VK_VEC + 4 * u + 0] = s4.x;
-          sc[ks * VK_VEC + 4 * u + 1] = s4.y;
-          sc[ks * VK_VEC + 4 * u + 2] = s4.z;
-          sc[ks * VK_VEC + 4 * u + 3] = s4.w;
-        }
-      }
-      // ---- mask, running max ----
-      bool vis[S_PER_LANE];
-      float tmax = -INFINITY;
-      int any = 0;
-#pragma unroll
-      for (int i = 0; i < S_PER_LANE; ++i) {
-        const int key = kb + (i / VK_VEC) * VK_SLAB + g * VK_VEC + (i % VK_VEC);
-        vis[i] = row_ok && key >= lo && key <= pos;
-        sc[i] = sc[i] * a.scale_log2;
-        tmax = fmaxf(tmax, vis[i] ? sc[i] : -INFINITY);
-        any |= vis[i] ? 1 : 0;
-      }
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, VK_WAVE));
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, VK_WAVE));
-      any |= __shfl_xor(any, 16, VK_WAVE);
-      any |= __shfl_xor(any, 32, VK_WAVE);
-      const float m_new = any ? fmaxf(m_run, tmax) : m_run;
-      const float alpha = any ? fast_exp2(m_run - m_new) : 1.0f;
-      float psum = 0.f;
-      float pr[S_PER_LANE];
-#pragma unroll
-      for (int i = 0; i < S_PER_LANE; ++i) {
-        pr[i] = vis[i] ? fast_exp2(sc[i] - m_new) : 0.f;
-        psum = psum + pr[i];
-      }
-      psum = psum + __shfl_xor(psum, 16, VK_WAVE);
-      psum = psum + __shfl_xor(psum, 32, VK_WAVE);
-      l_run = any ? l_run * alpha + psum : l_run;
-      m_run = m_new;
-      // ---- P fragments (second operand of O^T = V^T P^T), rounded to the element type ----
-      frag_t pf[KEY_SLABS];
-#pragma unroll
-      for (int ks = 0; ks < KEY_SLABS; ++ks) {
-#ifdef VK_BF16
-#pragma unroll
-        for (int j = 0; j < 8; ++j) pf[ks][j] = (__bf16)pr[ks * 8 + j];
-#else
-        pf[ks] = f32x4{pr[ks * 4 + 0], pr[ks * 4 + 1], pr[ks * 4 + 2], pr[ks * 4 + 3]};
-#endif
-      }
-      // ---- acc = acc * alpha + V^T P^T ----
-      // Keys outside [wave_lo, k_len) may lie in pages this sequence does not own
-      // (never written, or given back once the window passed them): their values
-      // are replaced by zero so that stale NaN or Inf cannot reach the sum.
-      const bool edge = kb + TILE_KEYS > k_len || kb < wave_lo;
-#pragma unroll
-      for (int dt = 0; dt < NDT; ++dt) {
-        if (dt * 16 < d) {
-          acc[dt].x = acc[dt].x * alpha; acc[dt].y = acc[dt].y * alpha;
-          acc[dt].z = acc[dt].z * alpha; acc[dt].w = acc[dt].w * alpha;
-#pragma unroll
-          for (int ks = 0; ks < KEY_SLABS; ++ks) {
-            const int k0 = kb + ks * VK_SLAB + g * VK_VEC;
-            const bool vok = k0 < k_len;
-            const int kk = vok ? k0 : 0;
-            const int page = bt[kk / P];
-            const elem_t* vrow = vbase + page * page_stride + (int64_t)(dt * 16 + r16) * P + (kk % P);
-            frag_t vf = load_frag(vrow, vok);
-            if (edge) {
-#pragma unroll
-              for (int j = 0; j < VK_VEC; ++j)
-                if (k0 + j >= k_len || k0 + j < wave_lo) vf[j] = (elem_t)0.f;
-            }
-            acc[dt] = mma_slab(vf, pf[ks], acc[dt]);
-          }
-        }
-      }
+    for (int dt = 0; dt < NDT; ++dt) As[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    const int t_end = min(tile_hi, seg * SEG_TILES + SEG_TILES - 1);
+    for (int t = max(tile_lo, seg * SEG_TILES); t <= t_end; ++t) {
+      float m_t, l_t;
+      f32x4 acc[NDT];
+      tile_partial<NDT, NQS>(c, qf, t * TILE_KEYS, m_t, l_t, acc);
+      fold<NDT>(Ms, Ls, As, m_t, l_t, acc);
     }
-    // ---- leave the segment ----
-    if (SPLIT) {
-      if (row_ok) {
-        const int64_t prow = ((int64_t)tok * a.nq + head) * a.nseg + seg;
-        if (g == 0) {
-          a.part_ml[2 * prow] = m_run;
-          a.part_ml[2 * prow + 1] = l_run;
-        }
-        if (m_run > -INFINITY) {
-#pragma unroll
-          for (int dt = 0; dt < NDT; ++dt)
-            if (dt * 16 < d) *reinterpret_cast<f32x4*>(a.part_acc + prow * d + dt * 16 + 4 * g) = acc[dt];
-        }
-      }
-    } else if (m_run > -INFINITY) {
-      const float Mn = fmaxf(M_tot, m_run);
-      const float ca = fast_exp2(M_tot - Mn), cb = fast_exp2(m_run - Mn);
-#pragma unroll
-      for (int dt = 0; dt < NDT; ++dt) {
-        ACC[dt].x = ACC[dt].x * ca + acc[dt].x * cb; ACC[dt].y = ACC[dt].y * ca + acc[dt].y * cb;
-        ACC[dt].z = ACC[dt].z * ca + acc[dt].z * cb; ACC[dt].w = ACC[dt].w * ca + acc[dt].w * cb;
-      }
-      L_tot = L_tot * ca + l_run * cb;
-      M_tot = Mn;
-    }
+    fold<NDT>(M, L, ACC, Ms, Ls, As);
   }
-  if (!SPLIT && row_ok) {
-    const float inv = L_tot > 0.f ? 1.0f / L_tot : 0.f;
-    elem_t* orow = a.out + ((int64_t)tok * a.nq + head) * d;
+  if (c.row_ok) {
+    const float inv = L > 0.f ? 1.0f / L : 0.f;
+    elem_t* orow = a.out + ((int64_t)tok * a.nq + head) * a.d;
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt) {
-      if (dt * 16 < d) {
+      if (dt * 16 < a.d) {
         const float o[4] = {ACC[dt].x * inv, ACC[dt].y * inv, ACC[dt].z * inv, ACC[dt].w * inv};
-        elem_t* p = orow + dt * 16 + 4 * g;
+        elem_t* p = orow + dt * 16 + 4 * c.g;
 #pragma unroll
         for (int i = 0; i < 4; ++i) p[i] = from_f32<elem_t>(o[i]);
       }
@@ -270,7 +288,85 @@ __global__ __launch_bounds__(64) void attn_kernel(AttnArgs a) {
   }
 }
 
-// Merges the segment results of one (token, head) in ascending segment order.
+// Decoded tokens: an item is one token; the 16 rows of a wave are up to 16 q
+// heads of one kv head.  Workgroup = one segment, wave = one tile of it.
+template <int DPAD>
+__global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
+  constexpr int NDT = DPAD / 16, NQS = DPAD / VK_SLAB;
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  float (*s_acc)[16][DPAD] = reinterpret_cast<float (*)[16][DPAD]>(smem);
+  float (*s_ml)[16][2] = reinterpret_cast<float (*)[16][2]>(smem + SEG_TILES * 16 * DPAD);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int G = a.nq / a.nkv, HT = (G + 15) >> 4;
+  const int kvh = blockIdx.y / HT, ht = blockIdx.y - kvh * HT;
+  const int seg = blockIdx.z;
+  const int seq = a.items[2 * blockIdx.x], q_off = a.items[2 * blockIdx.x + 1];
+  const int q_begin = a.cu_q[seq], q_len = a.cu_q[seq + 1] - q_begin;
+  const int k_len = a.k_len[seq];
+  const int tok = q_begin + q_off;
+  const int pos = k_len - q_len + q_off;
+  const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+  const int tile_lo = lo / TILE_KEYS, tile_hi = pos / TILE_KEYS;
+  if (seg < tile_lo / SEG_TILES || seg > tile_hi / SEG_TILES) return;   // whole workgroup
+
+  RowCtx c;
+  init_ctx(c, a, seq, kvh, k_len);
+  c.r16 = lane & 15;
+  c.g = lane >> 4;
+  const int nvalid = min(16, G - ht * 16);
+  c.row_ok = c.r16 < nvalid;
+  c.pos = pos;
+  c.lo = lo;
+  c.wave_lo = lo;
+  const int head = kvh * G + ht * 16 + c.r16;
+  const int t = seg * SEG_TILES + wave;
+  float m_t = -INFINITY, l_t = 0.f;
+  if (t >= tile_lo && t <= tile_hi) {
+    frag_t qf[NQS];
+    load_q<NQS>(a, tok, head, c.row_ok, c.g, qf);
+    f32x4 acc[NDT];
+    tile_partial<NDT, NQS>(c, qf, t * TILE_KEYS, m_t, l_t, acc);
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt)
+      if (dt * 16 < a.d) *reinterpret_cast<f32x4*>(&s_acc[wave][c.r16][dt * 16 + 4 * c.g]) = acc[dt];
+  }
+  if (c.g == 0) {
+    s_ml[wave][c.r16][0] = m_t;
+    s_ml[wave][c.r16][1] = l_t;
+  }
+  __syncthreads();
+  // Fold the segment's tiles: thread (row, column group) owns DPAD/16 columns.
+  const int row = threadIdx.x >> 4, cg = threadIdx.x & 15;
+  if (row >= nvalid) return;
+  float M = -INFINITY, L = 0.f;
+  float ACC[NDT];
+#pragma unroll
+  for (int i = 0; i < NDT; ++i) ACC[i] = 0.f;
+#pragma unroll
+  for (int w = 0; w < SEG_TILES; ++w) {
+    const float m = s_ml[w][row][0], l = s_ml[w][row][1];
+    if (m > -INFINITY) {
+      float Mn, ca, cb;
+      fold_scales(M, m, Mn, ca, cb);
+#pragma unroll
+      for (int i = 0; i < NDT; ++i) ACC[i] = fold1(ACC[i], s_acc[w][row][cg * NDT + i], ca, cb);
+      L = fold1(L, l, ca, cb);
+      M = Mn;
+    }
+  }
+  const int64_t prow = ((int64_t)tok * a.nq + (kvh * G + ht * 16 + row)) * a.nseg + seg;
+  if (cg == 0) {
+    a.part_ml[2 * prow] = M;
+    a.part_ml[2 * prow + 1] = L;
+  }
+  if (M > -INFINITY) {
+#pragma unroll
+    for (int i = 0; i < NDT; ++i)
+      if (cg * NDT + i < a.d) a.part_acc[prow * a.d + cg * NDT + i] = ACC[i];
+  }
+}
+
+// Folds the segment results of one (token, head) in ascending segment order.
 // One wave per row; lane j owns output columns j, j+64, ...
 __global__ __launch_bounds__(64) void attn_combine_kernel(AttnArgs a) {
   const int seq = a.items[2 * blockIdx.x], q_off = a.items[2 * blockIdx.x + 1];
@@ -282,42 +378,35 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(AttnArgs a) {
   const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
   const int seg_begin = lo / (TILE_KEYS * SEG_TILES), seg_end = pos / (TILE_KEYS * SEG_TILES) + 1;
   const int d = a.d;
-  float M_tot = -INFINITY, L_tot = 0.f;
+  float M = -INFINITY, L = 0.f;
   float ACC[4] = {0.f, 0.f, 0.f, 0.f};   // d <= 256
   const int64_t row0 = ((int64_t)tok * a.nq + head) * a.nseg;
   for (int seg = seg_begin; seg < seg_end; ++seg) {
-    const float m_run = a.part_ml[2 * (row0 + seg)], l_run = a.part_ml[2 * (row0 + seg) + 1];
-    if (m_run > -INFINITY) {
-      const float Mn = fmaxf(M_tot, m_run);
-      const float ca = fast_exp2(M_tot - Mn), cb = fast_exp2(m_run - Mn);
+    const float m = a.part_ml[2 * (row0 + seg)], l = a.part_ml[2 * (row0 + seg) + 1];
+    if (m > -INFINITY) {
+      float Mn, ca, cb;
+      fold_scales(M, m, Mn, ca, cb);
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int c = threadIdx.x + 64 * i;
-        if (c < d) ACC[i] = ACC[i] * ca + a.part_acc[(row0 + seg) * d + c] * cb;
+        const int col = threadIdx.x + 64 * i;
+        if (col < d) ACC[i] = fold1(ACC[i], a.part_acc[(row0 + seg) * d + col], ca, cb);
       }
-      L_tot = L_tot * ca + l_run * cb;
-      M_tot = Mn;
+      L = fold1(L, l, ca, cb);
+      M = Mn;
     }
   }
-  const float inv = L_tot > 0.f ? 1.0f / L_tot : 0.f;
+  const float inv = L > 0.f ? 1.0f / L : 0.f;
   elem_t* orow = a.out + ((int64_t)tok * a.nq + head) * d;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int c = threadIdx.x + 64 * i;
-    if (c < d) orow[c] = from_f32<elem_t>(ACC[i] * inv);
+    const int col = threadIdx.x + 64 * i;
+    if (col < d) orow[col] = from_f32<elem_t>(ACC[i] * inv);
   }
-}
-
-template <int MODE, bool SPLIT>
-static void launch_attn(int dpad, dim3 grid, const AttnArgs& a, hipStream_t st) {
-  if (dpad <= 64) attn_kernel<64, MODE, SPLIT><<<grid, 64, 0, st>>>(a);
-  else if (dpad <= 128) attn_kernel<128, MODE, SPLIT><<<grid, 64, 0, st>>>(a);
-  else attn_kernel<256, MODE, SPLIT><<<grid, 64, 0, st>>>(a);
 }
 
 extern "C" {
 
-// Number of floats of scratch a split launch needs for `tokens` rows.
+// Number of floats of scratch a decode launch needs for `tokens` rows.
 int64_t vk_attn_scratch_floats(int tokens, int nq, int d, int nseg) {
   const int64_t rows = (int64_t)tokens * nq * nseg;
   return ((rows * 2 + 3) & ~(int64_t)3) + rows * d;
@@ -326,22 +415,19 @@ int64_t vk_attn_scratch_floats(int tokens, int nq, int d, int nseg) {
 int vk_attn_segment_keys(void) { return TILE_KEYS * SEG_TILES; }
 
 // items: n_items pairs (sequence, first row).  mode 0: each item is up to 16
-// consecutive rows of the sequence's q_len new tokens, fused over segments.
-// mode 1: each item is one token; with split != 0 the keys are split by segment
-// over nseg workgroups (scratch must hold vk_attn_scratch_floats(T, ...)) and
-// merged by a second kernel.  The result is the same in every mode.
+// consecutive rows of the sequence's q_len new tokens.  mode 1: each item is one
+// token; the keys are split by segment over nseg workgroups (nseg must cover
+// the longest sequence; scratch must hold vk_attn_scratch_floats(T, ...)) and
+// folded by a second kernel.  The result is the same in both modes.
 int vk_paged_attention(elem_t* out, const elem_t* q, const elem_t* kc, const elem_t* vc,
                        const int32_t* block_table, int bt_stride, const int32_t* cu_q, const int32_t* k_len,
-                       const int32_t* items, int n_items, int mode, int split, int nseg, float* scratch,
-                       int total_tokens, int nq, int nkv, int d, int P, int window, float scale,
-                       hipStream_t st) {
+                       const int32_t* items, int n_items, int mode, int nseg, float* scratch, int total_tokens,
+                       int nq, int nkv, int d, int P, int window, float scale, hipStream_t st) {
   VK_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0, "attention: %d q heads are not a multiple of %d kv heads", nq, nkv);
   VK_REQUIRE(d >= 16 && d <= 256 && d % 16 == 0, "attention: head size %d must be a multiple of 16 in 16..256", d);
   VK_REQUIRE(P >= 8 && (P & (P - 1)) == 0, "attention: page size %d must be a power of two >= 8", P);
   VK_REQUIRE(window >= 0, "attention: window %d must not be negative", window);
   VK_REQUIRE(mode == 0 || mode == 1, "attention: unknown mode %d", mode);
-  VK_REQUIRE(!(split && mode == 0), "attention: split is for single-token items only");
-  VK_REQUIRE(nq <= 65535, "attention: too many heads");
   if (n_items <= 0) return 0;
   AttnArgs a;
   a.q = q; a.out = out; a.kc = kc; a.vc = vc; a.block_table = block_table; a.cu_q = cu_q; a.k_len = k_len;
@@ -350,18 +436,34 @@ int vk_paged_attention(elem_t* out, const elem_t* q, const elem_t* kc, const ele
   a.part_ml = nullptr; a.part_acc = nullptr;
   const int G = nq / nkv;
   if (mode == 0) {
-    launch_attn<0, false>(d, dim3(n_items, nq, 1), a, st);
-  } else if (!split) {
-    launch_attn<1, false>(d, dim3(n_items, nkv * ((G + 15) / 16), 1), a, st);
-  } else {
-    VK_REQUIRE(nseg > 0 && nseg <= 65535 && scratch != nullptr, "attention: split needs nseg in 1..65535 and scratch");
-    a.part_ml = scratch;
-    a.part_acc = scratch + (((int64_t)total_tokens * nq * nseg * 2 + 3) & ~(int64_t)3);
-    launch_attn<1, true>(d, dim3(n_items, nkv * ((G + 15) / 16), nseg), a, st);
-    if (vk_check_launch("attention")) return 1;
-    attn_combine_kernel<<<dim3(n_items, nq), 64, 0, st>>>(a);
+    const int hpw = G < 4 ? G : 4;
+    const dim3 grid(n_items, nkv * ((G + hpw - 1) / hpw));
+    VK_REQUIRE(grid.y <= 65535, "attention: too many heads");
+    if (d <= 64) attn_prefill_kernel<64><<<grid, 64 * hpw, 0, st>>>(a, hpw);
+    else if (d <= 128) attn_prefill_kernel<128><<<grid, 64 * hpw, 0, st>>>(a, hpw);
+    else attn_prefill_kernel<256><<<grid, 64 * hpw, 0, st>>>(a, hpw);
+    return vk_check_launch("attention (prompt rows)");
   }
-  return vk_check_launch("attention");
+  VK_REQUIRE(nseg > 0 && nseg <= 65535 && scratch != nullptr, "attention: decode needs nseg in 1..65535 and scratch");
+  a.part_ml = scratch;
+  a.part_acc = scratch + (((int64_t)total_tokens * nq * nseg * 2 + 3) & ~(int64_t)3);
+  const dim3 grid(n_items, nkv * ((G + 15) / 16), nseg);
+  VK_REQUIRE(grid.y <= 65535 && nq <= 65535, "attention: too many heads");
+#define DECODE(DP)                                                                                   \
+  do {                                                                                               \
+    const size_t smem = (size_t)SEG_TILES * 16 * (DP + 2) * sizeof(float);                           \
+    if (smem > 48 * 1024)                                                                            \
+      (void)hipFuncSetAttribute((const void*)attn_decode_kernel<DP>,                                 \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);              \
+    attn_decode_kernel<DP><<<grid, 256, smem, st>>>(a);                                              \
+  } while (0)
+  if (d <= 64) DECODE(64);
+  else if (d <= 128) DECODE(128);
+  else DECODE(256);
+#undef DECODE
+  if (vk_check_launch("attention (decoded rows)")) return 1;
+  attn_combine_kernel<<<dim3(n_items, nq), 64, 0, st>>>(a);
+  return vk_check_launch("attention (combine)");
 }
 
 }  // extern "C"

@@ -12,9 +12,12 @@
 // for the same reason (kernels/triton_kernels/matmul.py:33-73,
 // kernels/triton_kernels/qkv_matmul.py:24-32).
 //
-//   gemm_skinny: M <= 64.  Streams the weights once from HBM; a workgroup of
-//                eight waves owns 16*NTW weight rows and the waves split K by
-//                chunk.  Chunk sums meet in LDS and are added in chunk order.
+//   gemm_skinny: M <= 64.  Streams the weights once from HBM.  A workgroup of
+//                eight waves owns 16 weight rows; wave w takes the chunks w,
+//                w+8, ... and keeps a rolling window of W slabs (weights and
+//                activations) in flight, also across chunk borders.  After each
+//                round of eight chunks the chunk sums meet in LDS and are added
+//                in chunk order.
 //   gemm_tiled:  any M.  128x128 output tile per workgroup staged through LDS,
 //                64x64 per wave; a second accumulator set holds the total.
 #include "common.h"
@@ -23,6 +26,7 @@
 
 #define KC 512                        // elements per chunk
 #define KC_SLABS (KC / VK_SLAB)       // 16 (bfloat16) or 32 (float)
+#define SK_WAVES 8
 
 __device__ __forceinline__ void store_out4(elem_t* out, int64_t ldo, int m, int n, int M, int N, f32x4 v,
                                            bool vec_ok) {
@@ -45,94 +49,73 @@ __device__ __forceinline__ void store_out4(elem_t* out, int64_t ldo, int m, int 
 }
 
 // ------------------------------------------------------------------ skinny
-template <int NTW, int MT>
-__global__ __launch_bounds__(512) void gemm_skinny_kernel(elem_t* __restrict__ out, const elem_t* __restrict__ act,
-                                                          const elem_t* __restrict__ w, int M, int N, int K,
-                                                          int64_t lda, int64_t ldo, int out_vec_ok) {
-  constexpr int ITEMS = NTW * MT;
-  constexpr int SL = 16 / NTW;            // slabs per stage (a stage is 16 weight fragments)
-  constexpr int NST = KC_SLABS / SL;      // stages per chunk
-  __shared__ f32x4 part[8][ITEMS][64];
+// MT: 16-row activation tiles (M <= 16*MT).  W: slabs in flight per wave.
+template <int MT, int W>
+__global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_kernel(elem_t* __restrict__ out,
+                                                                    const elem_t* __restrict__ act,
+                                                                    const elem_t* __restrict__ w, int M, int N, int K,
+                                                                    int64_t lda, int64_t ldo, int out_vec_ok) {
+  static_assert(KC_SLABS % W == 0, "the window must divide a chunk");
+  __shared__ f32x4 part[SK_WAVES][MT][64];
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r16 = lane & 15, kg = lane >> 4;
-  const int n0 = blockIdx.x * (16 * NTW);
+  const int n0 = blockIdx.x * 16;
   const int nchunks = (K + KC - 1) / KC;
-  const int rounds = (nchunks + 7) / 8;
+  const int rounds = (nchunks + SK_WAVES - 1) / SK_WAVES;
 
-  const elem_t* wrow[NTW];
-  bool wok[NTW];
-#pragma unroll
-  for (int nt = 0; nt < NTW; ++nt) {
-    const int n = n0 + nt * 16 + r16;
-    wok[nt] = n < N;
-    wrow[nt] = w + (int64_t)(wok[nt] ? n : 0) * K;
-  }
+  const bool wok = n0 + r16 < N;
+  const elem_t* wrow = w + (int64_t)(wok ? n0 + r16 : 0) * K + kg * VK_VEC;
   const elem_t* arow[MT];
   bool aok[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int m = mt * 16 + r16;
     aok[mt] = m < M;
-    arow[mt] = act + (int64_t)(aok[mt] ? m : 0) * lda;
+    arow[mt] = act + (int64_t)(aok[mt] ? m : 0) * lda + kg * VK_VEC;
   }
 
+  frag_t wbuf[W], abuf[W][MT];
+  auto issue = [&](int c, int s, int slot) {
+    const int k = c * KC + s * VK_SLAB;
+    const bool kok = k + kg * VK_VEC < K;
+    wbuf[slot] = load_frag(wrow + k, wok && kok);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) abuf[slot][mt] = load_frag(arow[mt] + k, aok[mt] && kok);
+  };
+
+  int c = wave;
+  if (c < nchunks) {
+#pragma unroll
+    for (int i = 0; i < W; ++i) issue(c, i, i);
+  }
   f32x4 total = {0.f, 0.f, 0.f, 0.f};
-
-  for (int round = 0; round < rounds; ++round) {
-    const int c = round * 8 + wave;
-    f32x4 acc[NTW][MT];
+  for (int round = 0; round < rounds; ++round, c += SK_WAVES) {
+    f32x4 acc[MT];
 #pragma unroll
-    for (int nt = 0; nt < NTW; ++nt)
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-
+    for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
     if (c < nchunks) {
-      const int kbase = c * KC + kg * VK_VEC;
-      frag_t cur[16], nxt[16];
+      const int cn = c + SK_WAVES;
+      const bool has_next = cn < nchunks;
 #pragma unroll
-      for (int sl = 0; sl < SL; ++sl)
+      for (int i = 0; i < KC_SLABS; ++i) {
+        const int slot = i % W;
+        const frag_t fw = wbuf[slot];
+        frag_t fa[MT];
 #pragma unroll
-        for (int nt = 0; nt < NTW; ++nt) {
-          const int k = kbase + sl * VK_SLAB;
-          cur[sl * NTW + nt] = load_frag(wrow[nt] + k, wok[nt] && k < K);
-        }
+        for (int mt = 0; mt < MT; ++mt) fa[mt] = abuf[slot][mt];
+        if (i + W < KC_SLABS) issue(c, i + W, slot);
+        else if (has_next) issue(cn, i + W - KC_SLABS, slot);
 #pragma unroll
-      for (int st = 0; st < NST; ++st) {
-        if (st + 1 < NST) {
-#pragma unroll
-          for (int sl = 0; sl < SL; ++sl)
-#pragma unroll
-            for (int nt = 0; nt < NTW; ++nt) {
-              const int k = kbase + ((st + 1) * SL + sl) * VK_SLAB;
-              nxt[sl * NTW + nt] = load_frag(wrow[nt] + k, wok[nt] && k < K);
-            }
-        }
-#pragma unroll
-        for (int sl = 0; sl < SL; ++sl) {
-          const int k = kbase + (st * SL + sl) * VK_SLAB;
-          frag_t af[MT];
-#pragma unroll
-          for (int mt = 0; mt < MT; ++mt) af[mt] = load_frag(arow[mt] + k, aok[mt] && k < K);
-#pragma unroll
-          for (int nt = 0; nt < NTW; ++nt)
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = mma_slab(cur[sl * NTW + nt], af[mt], acc[nt][mt]);
-        }
-        if (st + 1 < NST) {
-#pragma unroll
-          for (int i = 0; i < 16; ++i) cur[i] = nxt[i];
-        }
+        for (int mt = 0; mt < MT; ++mt) acc[mt] = mma_slab(fw, fa[mt], acc[mt]);
       }
     }
 #pragma unroll
-    for (int nt = 0; nt < NTW; ++nt)
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) part[wave][nt * MT + mt][lane] = acc[nt][mt];
+    for (int mt = 0; mt < MT; ++mt) part[wave][mt][lane] = acc[mt];
     __syncthreads();
-    if (wave < ITEMS) {
-      for (int w2 = 0; w2 < 8; ++w2) {
-        if (round * 8 + w2 < nchunks) {
+    if (wave < MT) {
+      for (int w2 = 0; w2 < SK_WAVES; ++w2) {
+        if (round * SK_WAVES + w2 < nchunks) {
           const f32x4 p = part[w2][wave][lane];
           total.x = total.x + p.x; total.y = total.y + p.y; total.z = total.z + p.z; total.w = total.w + p.w;
         }
@@ -140,9 +123,100 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(elem_t* __restrict__ o
     }
     __syncthreads();
   }
-  if (wave < ITEMS) {
-    const int nt = wave / MT, mt = wave - nt * MT;
-    store_out4(out, ldo, mt * 16 + r16, n0 + nt * 16 + 4 * kg, M, N, total, out_vec_ok);
+  if (wave < MT) store_out4(out, ldo, wave * 16 + r16, n0 + 4 * kg, M, N, total, out_vec_ok);
+}
+
+// ---------------------------------------------------------------- streaming
+// The skinny kernel for K a multiple of 512, built to keep HBM busy: workgroups
+// are persistent and walk over weight tiles (16 rows) with a stride of the grid;
+// a wave's window of W slabs in flight runs on across tile borders, so the
+// memory pipe never drains; no load is predicated (rows beyond N or M are
+// clamped to the last valid row and their results dropped), because a select on
+// a loaded value makes the compiler wait for it at once; and with RES (K <= 4096,
+// one 16-row activation tile) a wave keeps the activations of its chunk in
+// registers for the whole kernel.  One barrier per round of eight chunks.
+template <int MT, int W, bool RES>
+__global__ __launch_bounds__(64 * SK_WAVES) void gemm_stream_kernel(elem_t* __restrict__ out,
+                                                                    const elem_t* __restrict__ act,
+                                                                    const elem_t* __restrict__ w, int M, int N, int K,
+                                                                    int64_t lda, int64_t ldo, int out_vec_ok) {
+  static_assert(KC_SLABS % W == 0, "the window must divide a chunk");
+  static_assert(!RES || MT == 1, "resident activations are for one activation tile");
+  __shared__ f32x4 part[2][SK_WAVES][MT][64];
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r16 = lane & 15, kg = lane >> 4;
+  const int nchunks = K / KC;
+  const int ntiles = (N + 15) / 16;
+
+  const elem_t* arow[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) arow[mt] = act + (int64_t)min(mt * 16 + r16, M - 1) * lda + kg * VK_VEC;
+
+  frag_t wbuf[W], abuf[RES ? KC_SLABS : W][MT];
+  if (RES) {
+    if (wave < nchunks) {
+#pragma unroll
+      for (int s = 0; s < KC_SLABS; ++s) abuf[s][0] = *reinterpret_cast<const frag_t*>(arow[0] + wave * KC + s * VK_SLAB);
+    }
+  }
+  auto issue = [&](int tile, int c, int s, int slot) {
+    const int k = c * KC + s * VK_SLAB;
+    wbuf[slot] = *reinterpret_cast<const frag_t*>(w + (int64_t)min(tile * 16 + r16, N - 1) * K + kg * VK_VEC + k);
+    if (!RES) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) abuf[slot][mt] = *reinterpret_cast<const frag_t*>(arow[mt] + k);
+    }
+  };
+
+  int tile = blockIdx.x;
+  if (tile < ntiles && wave < nchunks) {
+#pragma unroll
+    for (int i = 0; i < W; ++i) issue(tile, wave, i, i);
+  }
+  int parity = 0;
+  for (; tile < ntiles; tile += gridDim.x) {
+    f32x4 total = {0.f, 0.f, 0.f, 0.f};
+    for (int base = 0; base < nchunks; base += SK_WAVES) {
+      const int c = base + wave;
+      f32x4 acc[MT];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (c < nchunks) {
+        // What this wave streams next: its next chunk of this tile, else its first chunk of the next tile.
+        int nt = tile, nc = c + SK_WAVES;
+        if (nc >= nchunks) {
+          nt = tile + gridDim.x;
+          nc = wave;
+        }
+        const bool has_next = nt < ntiles;
+#pragma unroll
+        for (int i = 0; i < KC_SLABS; ++i) {
+          const int slot = i % W;
+          const frag_t fw = wbuf[slot];
+          frag_t fa[MT];
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) fa[mt] = RES ? abuf[i][mt] : abuf[slot][mt];
+          if (i + W < KC_SLABS) issue(tile, c, i + W, slot);
+          else if (has_next) issue(nt, nc, i + W - KC_SLABS, slot);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) acc[mt] = mma_slab(fw, fa[mt], acc[mt]);
+        }
+      }
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) part[parity][wave][mt][lane] = acc[mt];
+      __syncthreads();
+      if (wave < MT) {
+        for (int w2 = 0; w2 < SK_WAVES; ++w2) {
+          if (base + w2 < nchunks) {
+            const f32x4 p = part[parity][w2][wave][lane];
+            total.x = total.x + p.x; total.y = total.y + p.y; total.z = total.z + p.z; total.w = total.w + p.w;
+          }
+        }
+      }
+      parity ^= 1;
+    }
+    if (wave < MT) store_out4(out, ldo, wave * 16 + r16, tile * 16 + 4 * kg, M, N, total, out_vec_ok);
   }
 }
 
@@ -253,13 +327,6 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(elem_t* __restrict__ ou
 }
 
 // ==================================================================== host
-template <int NTW, int MT>
-static void launch_skinny(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K, int64_t lda,
-                          int64_t ldo, int vec_ok, hipStream_t st) {
-  const int per = 16 * NTW;
-  gemm_skinny_kernel<NTW, MT><<<(N + per - 1) / per, 512, 0, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok);
-}
-
 extern "C" {
 
 // kernel: 0 = choose by M, 1 = skinny (M <= 64), 2 = tiled.  The result does not
@@ -268,7 +335,6 @@ int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K
             int kernel, hipStream_t st) {
   VK_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
   VK_REQUIRE(K % VK_VEC == 0, "gemm: K=%d must be a multiple of %d for this element type", K, VK_VEC);
-  VK_REQUIRE(K <= 8 * 8 * KC, "gemm: K=%d exceeds the supported maximum of %d", K, 8 * 8 * KC);
   VK_REQUIRE(lda >= K && lda % VK_VEC == 0, "gemm: activation row stride %lld must be >= K and a multiple of %d",
              (long long)lda, VK_VEC);
   VK_REQUIRE(ldo >= N, "gemm: output row stride %lld is smaller than N=%d", (long long)ldo, N);
@@ -280,13 +346,35 @@ int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K
   if (kernel == 1) {
     VK_REQUIRE(M <= 64, "gemm: the skinny kernel takes at most 64 rows, got %d", M);
     const int mt = (M + 15) / 16;
-    int ntw = N >= 65536 ? 4 : (N >= 16384 ? 2 : 1);
-    while (ntw * mt > 4) ntw >>= 1;
-#define SK(NTW, MT) launch_skinny<NTW, MT>(out, act, w, M, N, K, lda, ldo, vec_ok, st)
-    if (mt == 1) { if (ntw == 4) SK(4, 1); else if (ntw == 2) SK(2, 1); else SK(1, 1); }
-    else if (mt == 2) { if (ntw == 2) SK(2, 2); else SK(1, 2); }
-    else if (mt == 3) SK(1, 3);
-    else SK(1, 4);
+    const unsigned grid = (unsigned)((N + 15) / 16);
+    if (K % KC == 0) {
+#define ST(MT, W, RES)                                                                                    \
+  do {                                                                                                    \
+    static int resident = 0; /* workgroups of this kernel that the device holds at once */               \
+    if (resident == 0) {                                                                                  \
+      int dev = 0, cus = 0, per_cu = 0;                                                                   \
+      (void)hipGetDevice(&dev);                                                                           \
+      (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);                      \
+      (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gemm_stream_kernel<MT, W, RES>,         \
+                                                         64 * SK_WAVES, 0);                               \
+      resident = (cus > 0 ? cus : 256) * (per_cu > 0 ? per_cu : 1);                                       \
+    }                                                                                                     \
+    gemm_stream_kernel<MT, W, RES><<<grid < (unsigned)resident ? grid : (unsigned)resident, 64 * SK_WAVES, \
+                                     0, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok);                    \
+  } while (0)
+      if (mt == 1) { if (K <= SK_WAVES * KC) ST(1, 8, true); else ST(1, 8, false); }
+      else if (mt == 2) ST(2, 8, false);
+      else if (mt == 3) ST(3, 4, false);
+      else ST(4, 4, false);
+#undef ST
+      return vk_check_launch("gemm_stream");
+    }
+#define SK(MT, W) gemm_skinny_kernel<MT, W><<<grid, 64 * SK_WAVES, 0, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok)
+    // Few weight rows leave one workgroup per compute unit: a deeper window keeps its memory pipe full.
+    if (mt == 1) { if (N <= 8192) SK(1, 16); else SK(1, 8); }
+    else if (mt == 2) SK(2, 8);
+    else if (mt == 3) SK(3, 4);
+    else SK(4, 4);
 #undef SK
     return vk_check_launch("gemm_skinny");
   }

@@ -2,14 +2,19 @@
 // python/vosti_kernels/kernels.py:1088-1104: argmax, first index on ties, a
 // NaN counts as the maximum) and temperature sampling by inverse CDF.
 //
-// One workgroup of 256 threads per row.  For temperature sampling thread t owns
-// the contiguous range [t*C, (t+1)*C) of the vocabulary, C = ceil(V/256): its
-// sum runs over the range in ascending order, the 256 sums are scanned serially
-// in thread order, and the owner of the target walks its range again.  The
-// result is a function of the row, the temperature and the uniform number only.
+// Two launches.  The first cuts every row into SAMPLE_BLOCKS contiguous ranges
+// and finds each range's maximum and its first index.  The second, one
+// workgroup of 1024 threads per row, merges them in range order; for
+// temperature sampling thread t then owns the contiguous range [t*C, (t+1)*C)
+// of the vocabulary, C = ceil(V/1024): its sum of exp((x - max)/T) runs over the
+// range in ascending order, the 1024 sums are scanned serially in thread order,
+// and the owner of the target walks its range again.  The result is a function
+// of the row, the temperature and the uniform number only.
 #include "common.h"
 
-#define SAMPLE_THREADS 256
+#define SAMPLE_BLOCKS 32
+#define PARTIAL_THREADS 256
+#define FINAL_THREADS 1024
 
 __device__ __forceinline__ bool better(float v, int i, float bv, int bi) {
   const bool vn = v != v, bn = bv != bv;
@@ -18,64 +23,83 @@ __device__ __forceinline__ bool better(float v, int i, float bv, int bi) {
   return v > bv || (v == bv && i < bi);
 }
 
-__global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(int32_t* __restrict__ out,
-                                                                const elem_t* __restrict__ logits,
-                                                                const float* __restrict__ temps,
-                                                                const float* __restrict__ uniforms, int V,
-                                                                int64_t row_stride) {
-  __shared__ float s_val[SAMPLE_THREADS];
-  __shared__ int s_idx[SAMPLE_THREADS];
-  __shared__ float s_pre[SAMPLE_THREADS + 1];
-  const int r = blockIdx.x, t = threadIdx.x;
+__global__ __launch_bounds__(PARTIAL_THREADS) void argmax_partial_kernel(float* __restrict__ pval, int* __restrict__ pidx,
+                                                                         const elem_t* __restrict__ logits, int V,
+                                                                         int64_t row_stride) {
+  __shared__ float s_val[PARTIAL_THREADS];
+  __shared__ int s_idx[PARTIAL_THREADS];
+  const int r = blockIdx.x, b = blockIdx.y, t = threadIdx.x;
   const elem_t* row = logits + r * row_stride;
-  const float temp = temps ? temps[r] : 0.f;
-
-  // ---- maximum and its first index ----
+  const int span = (V + SAMPLE_BLOCKS - 1) / SAMPLE_BLOCKS;
+  const int lo = min(V, b * span), hi = min(V, lo + span);
   float bv = -INFINITY;
   int bi = 0x7fffffff;
-  for (int i = t; i < V; i += SAMPLE_THREADS) {
+  for (int i = lo + t; i < hi; i += PARTIAL_THREADS) {
     const float v = to_f32(row[i]);
     if (better(v, i, bv, bi)) { bv = v; bi = i; }
   }
   s_val[t] = bv;
   s_idx[t] = bi;
   __syncthreads();
-  for (int off = SAMPLE_THREADS / 2; off > 0; off >>= 1) {
+  for (int off = PARTIAL_THREADS / 2; off > 0; off >>= 1) {
     if (t < off && better(s_val[t + off], s_idx[t + off], s_val[t], s_idx[t])) {
       s_val[t] = s_val[t + off];
       s_idx[t] = s_idx[t + off];
     }
     __syncthreads();
   }
-  const float vmax = s_val[0];
-  const int imax = s_idx[0];
+  if (t == 0) {
+    pval[r * SAMPLE_BLOCKS + b] = s_val[0];
+    pidx[r * SAMPLE_BLOCKS + b] = s_idx[0];
+  }
+}
+
+__global__ __launch_bounds__(FINAL_THREADS) void sample_final_kernel(int32_t* __restrict__ out,
+                                                                     const float* __restrict__ pval,
+                                                                     const int* __restrict__ pidx,
+                                                                     const elem_t* __restrict__ logits,
+                                                                     const float* __restrict__ temps,
+                                                                     const float* __restrict__ uniforms, int V,
+                                                                     int64_t row_stride) {
+  __shared__ float s_sum[FINAL_THREADS];
+  __shared__ float s_pre[FINAL_THREADS + 1];
+  __shared__ int s_owner;
+  const int r = blockIdx.x, t = threadIdx.x;
+  const elem_t* row = logits + r * row_stride;
+  const float temp = temps ? temps[r] : 0.f;
+  // Every thread merges the ranges' maxima in range order: the same result in all.
+  float vmax = -INFINITY;
+  int imax = 0x7fffffff;
+  for (int b = 0; b < SAMPLE_BLOCKS; ++b) {
+    const float v = pval[r * SAMPLE_BLOCKS + b];
+    const int i = pidx[r * SAMPLE_BLOCKS + b];
+    if (i != 0x7fffffff && better(v, i, vmax, imax)) { vmax = v; imax = i; }
+  }
   if (!(temp > 0.f) || vmax != vmax || vmax == INFINITY) {
     if (t == 0) out[r] = imax;
     return;
   }
   // ---- softmax(logits / temp) by inverse CDF ----
   const float zmax = vmax / temp;
-  const int C = (V + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
+  const int C = (V + FINAL_THREADS - 1) / FINAL_THREADS;
   const int lo = min(V, t * C), hi = min(V, lo + C);
   float sum = 0.f;
   for (int i = lo; i < hi; ++i) sum = sum + expf(to_f32(row[i]) / temp - zmax);
+  s_sum[t] = sum;
   __syncthreads();
-  s_val[t] = sum;
-  __syncthreads();
-  __shared__ int s_owner;
   if (t == 0) {
     float run = 0.f;
-    for (int j = 0; j < SAMPLE_THREADS; ++j) {
+    for (int j = 0; j < FINAL_THREADS; ++j) {
       s_pre[j] = run;
-      run = run + s_val[j];
+      run = run + s_sum[j];
     }
-    s_pre[SAMPLE_THREADS] = run;
+    s_pre[FINAL_THREADS] = run;
     // Owner: the first thread whose range carries the target; if rounding puts
     // the target at or beyond the total, the last thread with a positive sum.
     const float target0 = uniforms[r] * run;
     int own = -1, last = 0;
-    for (int j = 0; j < SAMPLE_THREADS; ++j) {
-      if (s_val[j] > 0.f) {
+    for (int j = 0; j < FINAL_THREADS; ++j) {
+      if (s_sum[j] > 0.f) {
         last = j;
         if (own < 0 && target0 < s_pre[j + 1]) own = j;
       }
@@ -83,9 +107,8 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(int32_t* __restr
     s_owner = own >= 0 ? own : last;
   }
   __syncthreads();
-  const float target = uniforms[r] * s_pre[SAMPLE_THREADS];
-  const bool owner = t == s_owner;
-  if (owner) {
+  if (t == s_owner) {
+    const float target = uniforms[r] * s_pre[FINAL_THREADS];
     float run = s_pre[t];
     int pick = -1, last_pos = lo;
     for (int i = lo; i < hi; ++i) {
@@ -100,14 +123,22 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(int32_t* __restr
 
 extern "C" {
 
+// Words (4 bytes each) of scratch that vk_sample needs for R rows.
+int vk_sample_scratch_words(int R) { return 2 * R * SAMPLE_BLOCKS; }
+
 // temps null: greedy for every row.  A row with temperature <= 0 is greedy.
-int vk_sample(int32_t* out, const elem_t* logits, const float* temps, const float* uniforms, int R, int V,
-              int64_t row_stride, hipStream_t st) {
+int vk_sample(int32_t* out, const elem_t* logits, const float* temps, const float* uniforms, void* scratch, int R,
+              int V, int64_t row_stride, hipStream_t st) {
   VK_REQUIRE(R >= 0 && V > 0, "sample: bad sizes R=%d V=%d", R, V);
   VK_REQUIRE(row_stride >= V, "sample: row stride %lld smaller than V=%d", (long long)row_stride, V);
   VK_REQUIRE(temps == nullptr || uniforms != nullptr, "sample: temperatures need uniform numbers");
+  VK_REQUIRE(scratch != nullptr, "sample: scratch is missing");
   if (R == 0) return 0;
-  sample_kernel<<<R, SAMPLE_THREADS, 0, st>>>(out, logits, temps, uniforms, V, row_stride);
+  float* pval = static_cast<float*>(scratch);
+  int* pidx = reinterpret_cast<int*>(pval + (int64_t)R * SAMPLE_BLOCKS);
+  argmax_partial_kernel<<<dim3(R, SAMPLE_BLOCKS), PARTIAL_THREADS, 0, st>>>(pval, pidx, logits, V, row_stride);
+  if (vk_check_launch("sample (partial)")) return 1;
+  sample_final_kernel<<<R, FINAL_THREADS, 0, st>>>(out, pval, pidx, logits, temps, uniforms, V, row_stride);
   return vk_check_launch("sample");
 }
 

@@ -15,7 +15,7 @@ import torch
 
 from . import build
 
-ABI_VERSION = 7
+ABI_VERSION = 9
 SEGMENT_KEYS = 256
 
 _DTYPES = {"bf16": torch.bfloat16, "f32": torch.float32}
@@ -66,8 +66,10 @@ class Kernels:
         _sig(lib.vk_fill_random, P, L, c_uint64, I, F, F, P)
         _sig(lib.vk_gemm, P, P, P, I, I, I, L, L, I, P)
         _sig(lib.vk_qkv_post, P, L, P, P, P, P, P, I, P, P, I, P, P, I, I, I, I, I, F, P)
-        _sig(lib.vk_paged_attention, P, P, P, P, P, I, P, P, P, I, I, I, I, P, I, I, I, I, I, I, F, P)
-        _sig(lib.vk_sample, P, P, P, P, I, I, L, P)
+        _sig(lib.vk_paged_attention, P, P, P, P, P, I, P, P, P, I, I, I, P, I, I, I, I, I, I, F, P)
+        _sig(lib.vk_sample, P, P, P, P, P, I, I, L, P)
+        lib.vk_sample_scratch_words.argtypes = [I]
+        lib.vk_sample_scratch_words.restype = c_int
         lib.vk_attn_scratch_floats.argtypes = [I, I, I, I]
         lib.vk_attn_scratch_floats.restype = c_int64
         lib.vk_attn_segment_keys.restype = c_int
@@ -255,7 +257,7 @@ class Kernels:
 
     def paged_attention(self, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                         block_table: torch.Tensor, cu_q: torch.Tensor, k_len: torch.Tensor, items: torch.Tensor,
-                        *, mode: int, scale: float, window: int = 0, max_k_len: int, split: bool = False,
+                        *, mode: int, scale: float, window: int = 0, max_k_len: int,
                         nseg: int = 0, scratch: torch.Tensor | None = None,
                         out: torch.Tensor | None = None) -> torch.Tensor:
         """Attention of the rows named by ``items`` over the paged cache (see attention.hip).
@@ -277,7 +279,7 @@ class Kernels:
         out = torch.empty_like(q) if out is None else out
         self._elem(out, "out", T, nq, d)
         sp = None
-        if split:
+        if mode == 1:
             need_seg = -(-max_k_len // SEGMENT_KEYS)
             if nseg < need_seg:
                 raise KernelError(f"attention: {nseg} segments do not cover {max_k_len} keys")
@@ -287,7 +289,7 @@ class Kernels:
             sp = self._f32(scratch, "scratch")
         self._call(self.lib.vk_paged_attention, out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                    block_table.data_ptr(), W, cu_q.data_ptr(), k_len.data_ptr(), items.data_ptr(), n_items, mode,
-                   1 if split else 0, nseg, sp, T, nq, nkv, d, P, window, float(scale), self._stream())
+                   nseg, sp, T, nq, nkv, d, P, window, float(scale), self._stream())
         return out
 
     def sample(self, logits: torch.Tensor, temps: torch.Tensor | None = None, uniforms: torch.Tensor | None = None,
@@ -300,7 +302,9 @@ class Kernels:
         tp = up = None
         if temps is not None:
             tp, up = self._f32(temps, "temps", R), self._f32(uniforms, "uniforms", R)
-        self._call(self.lib.vk_sample, out.data_ptr(), logits.data_ptr(), tp, up, R, V, V, self._stream())
+        scratch = torch.empty(self.lib.vk_sample_scratch_words(R), dtype=torch.int32, device=logits.device)
+        self._call(self.lib.vk_sample, out.data_ptr(), logits.data_ptr(), tp, up, scratch.data_ptr(), R, V, V,
+                   self._stream())
         return out
 
 
