@@ -58,6 +58,7 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=QWEN3_8B["num_hidden_layers"])
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--graphs", type=int, default=1, choices=[0, 1], help="replay decode steps from captured HIP graphs")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill timing")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -89,7 +90,7 @@ def main() -> int:
 
     def decode_run(B: int, steps: int, warmup: int):
         eng = Engine(model, num_pages=B * pages_per_request, page_size=page, max_num_seqs=B, max_num_batched_tokens=4096,
-                     enable_prefix_cache=False)
+                     enable_prefix_cache=False, graphs=bool(args.graphs))
         sp = SamplingParams(max_tokens=GENERATED_TOKENS, ignore_eos=True)
         for _ in range(B):
             eng.add_request(prompt(), sp)
@@ -137,7 +138,7 @@ def main() -> int:
                    "q_heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
                    "vocab_size": cfg.vocab_size, "global_batch": args.batch, "seq_len": PROMPT_TOKENS + GENERATED_TOKENS,
                    "prompt_tokens": PROMPT_TOKENS, "context_at_timing": round(ctx), "page_size": page,
-                   "parallelism": "single GPU", "graphs": False},
+                   "parallelism": "single GPU", "graphs": bool(args.graphs)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
     }

@@ -170,3 +170,18 @@ def test_smoke_entry():
     sys.path.insert(0, str(ROOT))
     import __graft_entry__
     __graft_entry__.smoke()
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_graph_replay_equals_eager(tiny_dirs, dtype_name):
+    """Decode steps replayed from captured graphs give the tokens of eager steps: several replays of
+    each graph, with eager prefill steps, arrivals and a growing block table between them."""
+    from vosti_amd.sampling import SamplingParams
+    ps = prompts("B", [3, 40, 17, 5], seed=12)
+    sp = [SamplingParams(max_tokens=60, temperature=0.7 * (i % 2), seed=i) for i in range(4)]
+    kw = dict(num_pages=64, page_size=8, max_num_seqs=3)
+    eager = engine(tiny_dirs["B"], dtype_name, **kw).generate(ps, sp, arrival_steps=[0, 0, 5, 30])
+    e = engine(tiny_dirs["B"], dtype_name, graphs=True, **kw)
+    assert e.generate(ps, sp, arrival_steps=[0, 0, 5, 30]) == eager
+    st = e.runner.graph_stats
+    assert st["captured"] >= 3 and st["replayed"] > 5 * st["captured"]

@@ -62,7 +62,7 @@ struct RowCtx {
   const elem_t* kbase;     // + kv head offset
   const elem_t* vbase;
   int64_t page_stride;
-  int k_len, d, P, r16, g;
+  int k_len, d, P, lp, r16, g;   // lp = log2(P)
   int lo, pos;             // this lane's row sees keys lo..pos
   int wave_lo;             // smallest key any row of the wave sees
   bool row_ok;
@@ -74,45 +74,40 @@ template <int NDT, int NQS>
 __device__ __forceinline__ void tile_partial(const RowCtx& c, const frag_t (&qf)[NQS], int kb, float& m_t, float& l_t,
                                              f32x4 (&acc)[NDT]) {
   const int d = c.d, P = c.P, r16 = c.r16, g = c.g;
-  // ---- scores S^T[key, row] = K Q^T ----
-  float sc[S_PER_LANE];
+  // No load below is predicated on data: addresses of keys beyond k_len are
+  // clamped to the last key (valid memory of this sequence) and what they bring
+  // is masked or zeroed later.  A select on a loaded value would make the
+  // compiler wait for every load right where it is issued.
+  const bool dfull = d % VK_SLAB == 0;    // else the last slab along d is partly outside the head
+  const int last_key = c.k_len - 1;
+  const int lp = c.lp;
+  // With pages of at least a tile, the tile lies in one page: one table lookup for the wave.
+  const bool one_page = P >= TILE_KEYS;
+  const int64_t tile_page = one_page ? (int64_t)c.bt[kb >> lp] * c.page_stride : 0;
+  const elem_t* kpage = c.kbase + tile_page;
+  const elem_t* vpage = c.vbase + tile_page;
+  // ---- key fragments of the whole tile, then value fragments, all in flight together ----
+  constexpr int KSUB = S_PER_LANE / 4;    // 16-key MFMA sub-tiles per tile
+  frag_t kf[KSUB][NQS];
 #pragma unroll
-  for (int ks = 0; ks < KEY_SLABS; ++ks) {
+  for (int sub = 0; sub < KSUB; ++sub) {
 #ifdef VK_BF16
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      // MFMA row m of this sub-tile is key  slab + 8*(m/4) + 4*u + m%4, so that
-      // lane group g ends up with the 8 consecutive keys slab + 8g .. 8g+7.
-      const int key = kb + ks * VK_SLAB + 8 * (r16 >> 2) + 4 * u + (r16 & 3);
+    // MFMA row m of sub-tile (ks, u) is key  slab + 8*(m/4) + 4*u + m%4, so that
+    // lane group g ends up with the 8 consecutive keys slab + 8g .. 8g+7.
+    const int key = kb + (sub >> 1) * VK_SLAB + 8 * (r16 >> 2) + 4 * (sub & 1) + (r16 & 3);
 #else
-    {
-      const int u = 0;
-      const int key = kb + ks * VK_SLAB + r16;
+    const int key = kb + sub * VK_SLAB + r16;
 #endif
-      const bool kok = key < c.k_len;
-      const int kk = kok ? key : 0;
-      const int page = c.bt[kk / P];
-      const elem_t* krow = c.kbase + page * c.page_stride + (int64_t)(kk % P) * d;
-      f32x4 s4 = {0.f, 0.f, 0.f, 0.f};
+    const int kk = min(key, last_key);
+    const elem_t* krow = (one_page ? kpage : c.kbase + c.bt[kk >> lp] * c.page_stride) + (int64_t)(kk & (P - 1)) * d;
 #pragma unroll
-      for (int s = 0; s < NQS; ++s) {
-        if (s * VK_SLAB < d) {
-          const int col = s * VK_SLAB + g * VK_VEC;
-          const frag_t kf = load_frag(krow + col, kok && col < d);
-          s4 = mma_slab(kf, qf[s], s4);
-        }
+    for (int s = 0; s < NQS; ++s) {
+      if (s * VK_SLAB < d) {
+        const int col = s * VK_SLAB + g * VK_VEC;
+        kf[sub][s] = dfull ? *reinterpret_cast<const frag_t*>(krow + col) : load_frag(krow + col, col < d);
       }
-      sc[ks * VK_VEC + 4 * u + 0] = s4.x;
-      sc[ks * VK_VEC + 4 * u + 1] = s4.y;
-      sc[ks * VK_VEC + 4 * u + 2] = s4.z;
-      sc[ks * VK_VEC + 4 * u + 3] = s4.w;
     }
   }
-  // ---- value fragments: requested before the softmax arithmetic needs them ----
-  // Keys outside [wave_lo, k_len) may lie in pages this sequence does not own
-  // (never written, or given back once the window passed them): their values
-  // are replaced by zero so that stale NaN or Inf cannot reach the sum.
-  const bool edge = kb + TILE_KEYS > c.k_len || kb < c.wave_lo;
   frag_t vf[NDT][KEY_SLABS];
 #pragma unroll
   for (int dt = 0; dt < NDT; ++dt) {
@@ -120,18 +115,25 @@ __device__ __forceinline__ void tile_partial(const RowCtx& c, const frag_t (&qf)
 #pragma unroll
       for (int ks = 0; ks < KEY_SLABS; ++ks) {
         const int k0 = kb + ks * VK_SLAB + g * VK_VEC;
-        const bool vok = k0 < c.k_len;
-        const int kk = vok ? k0 : 0;
-        const int page = c.bt[kk / P];
-        const elem_t* vrow = c.vbase + page * c.page_stride + (int64_t)(dt * 16 + r16) * P + (kk % P);
-        vf[dt][ks] = load_frag(vrow, vok);
-        if (edge) {
-#pragma unroll
-          for (int j = 0; j < VK_VEC; ++j)
-            if (k0 + j >= c.k_len || k0 + j < c.wave_lo) vf[dt][ks][j] = (elem_t)0.f;
-        }
+        const int kk = k0 <= last_key ? k0 : kb;     // a whole vector inside a page of this sequence
+        const elem_t* vrow = (one_page ? vpage : c.vbase + c.bt[kk >> lp] * c.page_stride) +
+                             (int64_t)(dt * 16 + r16) * P + (kk & (P - 1));
+        vf[dt][ks] = *reinterpret_cast<const frag_t*>(vrow);
       }
     }
+  }
+  // ---- scores S^T[key, row] = K Q^T ----
+  float sc[S_PER_LANE];
+#pragma unroll
+  for (int sub = 0; sub < KSUB; ++sub) {
+    f32x4 s4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < NQS; ++s)
+      if (s * VK_SLAB < d) s4 = mma_slab(kf[sub][s], qf[s], s4);
+    sc[4 * sub + 0] = s4.x;
+    sc[4 * sub + 1] = s4.y;
+    sc[4 * sub + 2] = s4.z;
+    sc[4 * sub + 3] = s4.w;
   }
   // ---- mask, maximum, probabilities ----
   bool vis[S_PER_LANE];
@@ -166,6 +168,23 @@ __device__ __forceinline__ void tile_partial(const RowCtx& c, const frag_t (&qf)
 #else
     pf[ks] = f32x4{pr[ks * 4 + 0], pr[ks * 4 + 1], pr[ks * 4 + 2], pr[ks * 4 + 3]};
 #endif
+  }
+  // Keys outside [wave_lo, k_len) may lie in pages this sequence does not own
+  // (never written, or given back once the window passed them): their values
+  // are replaced by zero so that stale NaN or Inf cannot reach the sum.
+  if (kb + TILE_KEYS > c.k_len || kb < c.wave_lo) {
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) {
+      if (dt * 16 < d) {
+#pragma unroll
+        for (int ks = 0; ks < KEY_SLABS; ++ks) {
+          const int k0 = kb + ks * VK_SLAB + g * VK_VEC;
+#pragma unroll
+          for (int j = 0; j < VK_VEC; ++j)
+            if (k0 + j >= c.k_len || k0 + j < c.wave_lo) vf[dt][ks][j] = (elem_t)0.f;
+        }
+      }
+    }
   }
 #pragma unroll
   for (int dt = 0; dt < NDT; ++dt) {
@@ -220,6 +239,7 @@ __device__ __forceinline__ void init_ctx(RowCtx& c, const AttnArgs& a, int seq, 
   c.k_len = k_len;
   c.d = a.d;
   c.P = a.P;
+  c.lp = __builtin_ctz(a.P);
   c.scale_log2 = a.scale_log2;
 }
 
@@ -381,18 +401,35 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(AttnArgs a) {
   float M = -INFINITY, L = 0.f;
   float ACC[4] = {0.f, 0.f, 0.f, 0.f};   // d <= 256
   const int64_t row0 = ((int64_t)tok * a.nq + head) * a.nseg;
-  for (int seg = seg_begin; seg < seg_end; ++seg) {
-    const float m = a.part_ml[2 * (row0 + seg)], l = a.part_ml[2 * (row0 + seg) + 1];
-    if (m > -INFINITY) {
-      float Mn, ca, cb;
-      fold_scales(M, m, Mn, ca, cb);
+  // Four segments are fetched together, then folded one after the other.
+  for (int seg0 = seg_begin; seg0 < seg_end; seg0 += 4) {
+    float m[4], l[4], v[4][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const bool in = seg0 + j < seg_end;
+      const int64_t r = row0 + (in ? seg0 + j : seg_begin);
+      m[j] = in ? a.part_ml[2 * r] : -INFINITY;
+      l[j] = a.part_ml[2 * r + 1];
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int64_t r = row0 + (seg0 + j < seg_end ? seg0 + j : seg_begin);
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int col = threadIdx.x + 64 * i;
-        if (col < d) ACC[i] = fold1(ACC[i], a.part_acc[(row0 + seg) * d + col], ca, cb);
+        v[j][i] = (col < d && m[j] > -INFINITY) ? a.part_acc[r * d + col] : 0.f;
       }
-      L = fold1(L, l, ca, cb);
-      M = Mn;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (m[j] > -INFINITY) {
+        float Mn, ca, cb;
+        fold_scales(M, m[j], Mn, ca, cb);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ACC[i] = fold1(ACC[i], v[j][i], ca, cb);
+        L = fold1(L, l[j], ca, cb);
+        M = Mn;
+      }
     }
   }
   const float inv = L > 0.f ? 1.0f / L : 0.f;

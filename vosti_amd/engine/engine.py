@@ -25,16 +25,17 @@ from .step import ModelRunner, StepEntry
 class Engine:
     def __init__(self, model: DecoderModel | str | Path, *, dtype="bfloat16", num_pages: int = 32, page_size: int = 64,
                  max_num_seqs: int = 8, max_num_batched_tokens: int = 4096, enable_prefix_cache: bool = True,
-                 max_model_len: int | None = None):
+                 max_model_len: int | None = None, graphs: bool = False):
         """``num_pages`` is the reference's VOSTI_NUM_BLOCKS (default 32 pages of 64 tokens),
         ``max_num_seqs`` VOSTI_MAX_SEQS and ``max_num_batched_tokens`` VOSTI_MAX_BATCHED_TOKENS
-        (examples/support/engine_setup.rs:57-69)."""
+        (examples/support/engine_setup.rs:57-69); ``graphs`` is VOSTI_CUDA_GRAPH: steps of decoded tokens
+        only are replayed from captured HIP graphs (engine_setup.rs:79-81)."""
         self.model = load_model(model, dtype) if isinstance(model, (str, Path)) else model
         self.kernels = self.model.kernels
         # One state slot per request that can be alive: those running plus the one being admitted.
         self.pool = CachePool(self.model, page_size=page_size, num_pages=num_pages, num_slots=max_num_seqs + 1,
                               prefix_cache=enable_prefix_cache)
-        self.runner = ModelRunner(self.model, self.pool)
+        self.runner = ModelRunner(self.model, self.pool, graphs=graphs)
         self.cache = self.pool.manager
         self.max_model_len = min(max_model_len or self.model.spec.max_positions, self.model.spec.max_positions)
         self.scheduler = Scheduler(self.cache, max_num_seqs, max_num_batched_tokens, self.max_model_len)

@@ -6,6 +6,13 @@ returns the logits at the places that are asked for.  The reference's
 counterpart is ``model_forward`` with the six step tensors
 (src/exec/model.rs:62-85, src/exec/cache_scheduler/mod.rs:824-930); here the
 wanted rows are arbitrary, not only each sequence's last.
+
+Steps that hold nothing but single decoded tokens, each wanting its logits, can
+be replayed from a captured HIP graph: the same forward pass, recorded once per
+(number of rows, block-table width) and fed through fixed device buffers.  The
+reference does the same around its forward (python/vosti_kernels/graph_overlay.py:177-389):
+a signature runs eagerly when first seen, is captured when seen again, and is
+replayed from then on.
 """
 from __future__ import annotations
 
@@ -15,9 +22,11 @@ import numpy as np
 import torch
 
 from ..cache import CachePool
+from ..kernels.ops import SEGMENT_KEYS
 from ..parts.base import GroupTables, StepContext
 
-ROW_TILE = 16   # rows of one attention work item
+ROW_TILE = 16          # rows of one attention work item
+WIDTH_BUCKET = 8       # captured block tables grow in steps of this many pages
 
 
 @dataclass
@@ -27,17 +36,51 @@ class StepEntry:
     want: list[int] = field(default_factory=list)   # places among ``tokens`` whose logits are wanted
 
 
+@dataclass
+class _Layout:
+    """Host arrays of one step and where each lies in the one buffer that is uploaded."""
+    parts: list[np.ndarray]
+    offsets: list[int]
+    total: int
+    q_lens: list[int]
+    starts: list[int]
+    max_k_len: int
+    max_decode_k_len: int
+
+    def pack(self, out: np.ndarray) -> None:
+        for p, o in zip(self.parts, self.offsets):
+            out[o:o + p.size] = p.reshape(-1)
+
+
+@dataclass
+class _Captured:
+    graph: torch.cuda.CUDAGraph
+    meta: torch.Tensor        # the device buffer the graph reads
+    staging: torch.Tensor     # pinned host twin
+    logits: torch.Tensor      # the graph's output
+    copied: torch.cuda.Event  # the last upload from ``staging``
+
+
 class ModelRunner:
     """Binds a model to a cache pool and runs steps."""
 
-    def __init__(self, model, pool: CachePool):
+    def __init__(self, model, pool: CachePool, graphs: bool = False):
         self.model, self.pool, self.cache = model, pool, pool.manager
         self.kernels = model.kernels
+        self.graphs = graphs
         self._scratch: torch.Tensor | None = None
+        self._seen: set[tuple] = set()
+        self._captured: dict[tuple, _Captured] = {}
+        self._keepalive: list[torch.Tensor] = []
+        self.graph_stats = {"eager": 0, "captured": 0, "replayed": 0}
 
     # ---------------------------------------------------------------- pieces
     def _attn_scratch(self, n_floats: int) -> torch.Tensor:
         if self._scratch is None or self._scratch.numel() < n_floats:
+            if torch.cuda.is_current_stream_capturing():
+                raise RuntimeError("the attention scratch buffer must be sized before a graph is captured")
+            if self._scratch is not None and self._captured:
+                self._keepalive.append(self._scratch)      # captured graphs still point at it
             self._scratch = torch.empty(max(n_floats, 1 << 16), dtype=torch.float32, device="cuda")
         return self._scratch
 
@@ -61,8 +104,8 @@ class ModelRunner:
         for e in entries:
             self.cache.commit(e.request_id)
 
-    def build_context(self, entries: list[StepEntry]) -> tuple[torch.Tensor, StepContext, torch.Tensor]:
-        """Host arrays of the step -> one upload -> (ids, context, wanted rows)."""
+    def _layout(self, entries: list[StepEntry], widths: list[int] | None = None) -> _Layout:
+        """The step's host arrays.  ``widths``: block-table width per group (default: what the step needs)."""
         cache, spec = self.cache, self.model.spec
         S = len(entries)
         q_lens = [len(e.tokens) for e in entries]
@@ -99,9 +142,8 @@ class ModelRunner:
                                    np.asarray(want, dtype=np.int32),
                                    np.asarray(prefill_items, dtype=np.int32).reshape(-1, 2),
                                    np.asarray(decode_items, dtype=np.int32).reshape(-1, 2)]
-        n_groups = len(self.pool.group_windows)
-        for g in range(n_groups):
-            width = max(1, max(cache.num_logical_pages(e.request_id, g) for e in entries))
+        for g in range(len(self.pool.group_windows)):
+            width = widths[g] if widths else self.needed_width(entries, g)
             table = np.zeros((S, width), dtype=np.int32)
             slots = np.empty(T, dtype=np.int32)
             for s, e in enumerate(entries):
@@ -113,25 +155,88 @@ class ModelRunner:
         for p in parts:
             offsets.append(total)
             total += (p.size + 3) & ~3
-        host = np.zeros(max(total, 4), dtype=np.int32)
-        for p, o in zip(parts, offsets):
-            host[o:o + p.size] = p.reshape(-1)
-        dev = torch.from_numpy(host).to("cuda")
-        views = [dev[o:o + p.size].view(p.shape) for p, o in zip(parts, offsets)]
-        ids_d, pos_d, cu_d, klen_d, slots_d, want_d, pre_d, dec_d = views[:8]
-        groups = [GroupTables(slots=views[8 + 2 * g], block_table=views[9 + 2 * g], window=self.pool.group_windows[g])
-                  for g in range(n_groups)]
         dec_k = [int(k_len[s]) for s, n in enumerate(q_lens) if n == 1]
-        ctx = StepContext(kernels=self.kernels, num_tokens=T, num_seqs=S, positions=pos_d, cu_q=cu_d, k_len=klen_d,
-                          state_slots=slots_d, groups=groups, prefill_items=pre_d, decode_items=dec_d,
-                          max_k_len=int(k_len.max()), max_decode_k_len=max(dec_k) if dec_k else 0,
-                          host_q_lens=q_lens, host_starts=starts, attn_scratch=self._attn_scratch)
+        return _Layout(parts, offsets, max(total, 4), q_lens, starts, int(k_len.max()), max(dec_k) if dec_k else 0)
+
+    def needed_width(self, entries: list[StepEntry], group: int) -> int:
+        return max(1, max(self.cache.num_logical_pages(e.request_id, group) for e in entries))
+
+    def _context(self, lay: _Layout, dev: torch.Tensor, max_k_len: int, max_decode_k_len: int):
+        views = [dev[o:o + p.size].view(p.shape) for p, o in zip(lay.parts, lay.offsets)]
+        ids_d, pos_d, cu_d, klen_d, slots_d, want_d, pre_d, dec_d = views[:8]
+        groups = [GroupTables(slots=views[8 + 2 * g], block_table=views[9 + 2 * g], window=w)
+                  for g, w in enumerate(self.pool.group_windows)]
+        ctx = StepContext(kernels=self.kernels, num_tokens=sum(lay.q_lens), num_seqs=len(lay.q_lens), positions=pos_d,
+                          cu_q=cu_d, k_len=klen_d, state_slots=slots_d, groups=groups, prefill_items=pre_d,
+                          decode_items=dec_d, max_k_len=max_k_len, max_decode_k_len=max_decode_k_len,
+                          host_q_lens=lay.q_lens, host_starts=lay.starts, host_state_slots=lay.parts[4].tolist(),
+                          attn_scratch=self._attn_scratch)
         return ids_d, ctx, want_d
 
+    def build_context(self, entries: list[StepEntry]):
+        """Host arrays of the step -> one upload -> (ids, context, wanted rows)."""
+        lay = self._layout(entries)
+        host = np.zeros(lay.total, dtype=np.int32)
+        lay.pack(host)
+        return self._context(lay, torch.from_numpy(host).to("cuda"), lay.max_k_len, lay.max_decode_k_len)
+
+    # ---------------------------------------------------------------- running
     def run(self, entries: list[StepEntry]) -> torch.Tensor:
         """The forward pass of a step whose pages are taken; logits [wanted, vocab] in the element type."""
+        if self.graphs and all(len(e.tokens) == 1 and e.want == [0] for e in entries):
+            return self._run_decode_graph(entries)
+        self.graph_stats["eager"] += 1
         ids, ctx, want = self.build_context(entries)
         return self.model.forward(ids, ctx, self.pool.entries, want)
+
+    def _run_decode_graph(self, entries: list[StepEntry]) -> torch.Tensor:
+        P = self.pool.page_size
+        widths = [-(-self.needed_width(entries, g) // WIDTH_BUCKET) * WIDTH_BUCKET
+                  for g in range(len(self.pool.group_windows))]
+        key = (len(entries), tuple(widths))
+        cap = self._captured.get(key)
+        if cap is None and key not in self._seen:
+            # First sight of a signature: eagerly, which also warms up every kernel it uses.
+            self._seen.add(key)
+            self.graph_stats["eager"] += 1
+            ids, ctx, want = self.build_context(entries)
+            return self.model.forward(ids, ctx, self.pool.entries, want)
+        lay = self._layout(entries, widths)
+        # Launch geometry is frozen in the graph: it must cover every length the tables can hold.
+        cover = min(max(widths) * P, self.model.spec.max_positions)
+        if cap is None:
+            T, spec = len(entries), self.model.spec
+            self._attn_scratch(self._max_scratch(T, cover))
+            staging = torch.empty(lay.total, dtype=torch.int32, pin_memory=True)
+            meta = torch.zeros(lay.total, dtype=torch.int32, device="cuda")
+            lay.pack(staging.numpy())
+            meta.copy_(staging, non_blocking=True)
+            ids, ctx, want = self._context(lay, meta, cover, cover)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                logits = self.model.forward(ids, ctx, self.pool.entries, want)
+            cap = _Captured(graph, meta, staging, logits, torch.cuda.Event())
+            self._captured[key] = cap
+            self.graph_stats["captured"] += 1
+        else:
+            cap.copied.synchronize()                       # the staging buffer is free again
+            lay.pack(cap.staging.numpy())
+            cap.meta.copy_(cap.staging, non_blocking=True)
+        cap.copied.record()
+        cap.graph.replay()
+        self.graph_stats["replayed"] += 1
+        return cap.logits
+
+    def _max_scratch(self, tokens: int, cover: int) -> int:
+        """Floats of attention scratch that any mixer of the model needs for ``tokens`` decode rows over ``cover`` keys."""
+        nseg = -(-cover // SEGMENT_KEYS)
+        need = 1
+        for block in self.model.layers:
+            m = block.mixer
+            if hasattr(m, "nq") and hasattr(m, "d"):
+                need = max(need, self.kernels.attn_scratch_floats(tokens, m.nq, m.d, nseg))
+        return need
 
     # ------------------------------------------------------------------ whole
     def step(self, entries: list[StepEntry]) -> torch.Tensor:

@@ -17,6 +17,7 @@ here; each also has a command-line option, which wins:
     VOSTI_NUM_BLOCKS           --num-blocks          cache pages (default 32)
     VOSTI_MAX_SEQS             --max-seqs            rows per step (default: the batch size)
     VOSTI_MAX_BATCHED_TOKENS   --max-batched-tokens  tokens per step (default 4096)
+    VOSTI_CUDA_GRAPH           --graphs              0/1: replay decode steps from captured HIP graphs
     VOSTI_OUTPUT_TOKENS        --output-tokens       write "index<TAB>ids" lines to this file
     VOSTI_BENCH_INPUT          --bench-input         TSV of MAX_TOKENS<TAB>IDS[<TAB>ARRIVAL_STEP] requests
     VOSTI_ENGINE_STEP_TRACE    --step-trace          append one JSON line per step to this file
@@ -56,6 +57,7 @@ def engine_parser() -> argparse.ArgumentParser:
     p.add_argument("--num-blocks", type=int, default=int(_env("VOSTI_NUM_BLOCKS", 32)))
     p.add_argument("--max-seqs", type=int, default=int(_env("VOSTI_MAX_SEQS", 0)))
     p.add_argument("--max-batched-tokens", type=int, default=int(_env("VOSTI_MAX_BATCHED_TOKENS", 4096)))
+    p.add_argument("--graphs", type=int, default=int(_env("VOSTI_CUDA_GRAPH", 0)), choices=[0, 1])
     p.add_argument("--output-tokens", default=_env("VOSTI_OUTPUT_TOKENS"))
     p.add_argument("--bench-input", default=_env("VOSTI_BENCH_INPUT"))
     p.add_argument("--step-trace", default=_env("VOSTI_ENGINE_STEP_TRACE"))
@@ -125,7 +127,7 @@ def run_engine(argv: list[str], family: str) -> int:
     eos = eos_ids(args.model_path)
     engine = Engine(args.model_path, dtype=args.dtype, num_pages=args.num_blocks, page_size=args.page_size,
                     max_num_seqs=args.max_seqs or len(requests), max_num_batched_tokens=args.max_batched_tokens,
-                    enable_prefix_cache=bool(args.prefix_cache))
+                    enable_prefix_cache=bool(args.prefix_cache), graphs=bool(args.graphs))
     params = [SamplingParams(max_tokens=m, temperature=args.temperature, seed=args.seed + i, eos_token_ids=eos,
                              ignore_eos=args.ignore_eos) for i, (m, _, _) in enumerate(requests)]
     trace = open(args.step_trace, "a") if args.step_trace else None
@@ -146,6 +148,8 @@ def run_engine(argv: list[str], family: str) -> int:
                                            "preemptions": engine.scheduler.preemptions()}, separators=(",", ":")))
     else:
         print(f"MODEL_OUTPUT_TOKEN_IDS={outputs[0]}")
+    if args.graphs:
+        print("GRAPH_STATS " + json.dumps(engine.runner.graph_stats, separators=(",", ":")))
     return 0
 
 

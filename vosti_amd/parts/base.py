@@ -114,6 +114,7 @@ class StepContext:
     max_decode_k_len: int
     host_q_lens: list[int] = field(default_factory=list)
     host_starts: list[int] = field(default_factory=list)   # position of each sequence's first token in this step
+    host_state_slots: list[int] = field(default_factory=list)   # host copy of ``state_slots``
     attn_scratch: Any = None     # callable(n_floats) -> float32 tensor
 
 
