@@ -377,3 +377,15 @@ def test_attention_refuses_bad_sizes():
     with pytest.raises(KernelError, match="head size"):
         k.paged_attention(q, kc, vc, i32(0, 1).view(1, 2), i32(0, 1), i32(1), i32(0, 0).view(1, 2), mode=1, scale=1.0,
                           max_k_len=1, nseg=1, scratch=torch.zeros(64, device="cuda"))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,I,K", [(8, 100, 1024), (16, 256, 4096), (1, 33, 512), (5, 48, 96), (20, 64, 1024)])
+def test_gemm_swiglu_fused_equals_separate(dtype, M, I, K):
+    """The gate/up projection with the activation folded in gives the bits of the two separate kernels
+    (the last two sizes fall back to them)."""
+    k = kern(dtype)
+    a, w = rand((M, K), dtype, 1).cuda(), rand((2 * I, K), dtype, 2, K ** -0.5).cuda()    # projections of order 1
+    got = k.gemm_swiglu(a, w)
+    assert torch.equal(got, k.swiglu(k.gemm(a, w, kernel=2)))
+    torch.testing.assert_close(got.float().cpu(), plain.swiglu(plain.linear(a.cpu(), w.cpu(), dtype), dtype), **tol(dtype))

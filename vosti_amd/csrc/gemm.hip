@@ -220,55 +220,266 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_stream_kernel(elem_t* __re
   }
 }
 
+// The streaming kernel for the gate/up projection with the activation folded in:
+// w holds I gate rows, then I up rows; a workgroup streams the gate tile and the
+// matching up tile together and writes  out[m, n] = silu(g) * u  with g and u the
+// two projections rounded to the element type first, which is what the separate
+// GEMM and SwiGLU kernels compute (kernels/triton_kernels/silu_mul.py:64-87).
+// M <= 16, K <= 4096 (activations resident in registers).
+template <int W>
+__global__ __launch_bounds__(64 * SK_WAVES) void gemm_stream_swiglu_kernel(elem_t* __restrict__ out,
+                                                                           const elem_t* __restrict__ act,
+                                                                           const elem_t* __restrict__ w, int M, int I,
+                                                                           int K, int64_t lda, int64_t ldo,
+                                                                           int out_vec_ok) {
+  static_assert(KC_SLABS % W == 0, "the window must divide a chunk");
+  __shared__ f32x4 part[2][SK_WAVES][2][64];
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r16 = lane & 15, kg = lane >> 4;
+  const int nchunks = K / KC;
+  const int ntiles = (I + 15) / 16;
+  const elem_t* arow = act + (int64_t)min(r16, M - 1) * lda + kg * VK_VEC;
+
+  frag_t wg[W], wu[W], abuf[KC_SLABS];
+  if (wave < nchunks) {
+#pragma unroll
+    for (int s = 0; s < KC_SLABS; ++s) abuf[s] = *reinterpret_cast<const frag_t*>(arow + wave * KC + s * VK_SLAB);
+  }
+  auto issue = [&](int tile, int s, int slot) {
+    const int64_t row = min(tile * 16 + r16, I - 1);
+    const elem_t* p = w + row * K + kg * VK_VEC + wave * KC + s * VK_SLAB;
+    wg[slot] = *reinterpret_cast<const frag_t*>(p);
+    wu[slot] = *reinterpret_cast<const frag_t*>(p + (int64_t)I * K);
+  };
+
+  int tile = blockIdx.x;
+  const bool active = wave < nchunks;
+  if (tile < ntiles && active) {
+#pragma unroll
+    for (int i = 0; i < W; ++i) issue(tile, i, i);
+  }
+  int parity = 0;
+  for (; tile < ntiles; tile += gridDim.x) {
+    f32x4 ag = {0.f, 0.f, 0.f, 0.f}, au = {0.f, 0.f, 0.f, 0.f};
+    if (active) {
+      const int nt = tile + gridDim.x;
+      const bool has_next = nt < ntiles;
+#pragma unroll
+      for (int i = 0; i < KC_SLABS; ++i) {
+        const int slot = i % W;
+        const frag_t fg = wg[slot], fu = wu[slot];
+        if (i + W < KC_SLABS) issue(tile, i + W, slot);
+        else if (has_next) issue(nt, i + W - KC_SLABS, slot);
+        ag = mma_slab(fg, abuf[i], ag);
+        au = mma_slab(fu, abuf[i], au);
+      }
+    }
+    part[parity][wave][0][lane] = ag;
+    part[parity][wave][1][lane] = au;
+    __syncthreads();
+    if (wave == 0) {
+      f32x4 tg = {0.f, 0.f, 0.f, 0.f}, tu = {0.f, 0.f, 0.f, 0.f};
+      for (int w2 = 0; w2 < nchunks; ++w2) {
+        const f32x4 pg = part[parity][w2][0][lane], pu = part[parity][w2][1][lane];
+        tg.x = tg.x + pg.x; tg.y = tg.y + pg.y; tg.z = tg.z + pg.z; tg.w = tg.w + pg.w;
+        tu.x = tu.x + pu.x; tu.y = tu.y + pu.y; tu.z = tu.z + pu.z; tu.w = tu.w + pu.w;
+      }
+      const float g[4] = {round_to_elem(tg.x), round_to_elem(tg.y), round_to_elem(tg.z), round_to_elem(tg.w)};
+      const float u[4] = {round_to_elem(tu.x), round_to_elem(tu.y), round_to_elem(tu.z), round_to_elem(tu.w)};
+      f32x4 y;
+      y.x = (g[0] * (1.0f / (1.0f + expf(-g[0])))) * u[0];
+      y.y = (g[1] * (1.0f / (1.0f + expf(-g[1])))) * u[1];
+      y.z = (g[2] * (1.0f / (1.0f + expf(-g[2])))) * u[2];
+      y.w = (g[3] * (1.0f / (1.0f + expf(-g[3])))) * u[3];
+      store_out4(out, ldo, r16, tile * 16 + 4 * kg, M, I, y, out_vec_ok);
+    }
+    parity ^= 1;
+  }
+}
+
 // ------------------------------------------------------------------- tiled
-#define T_BM 128
-#define T_BN 128
-#define T_ROWB 128                     // LDS bytes per tile row: two slabs; 16-byte columns are XOR-swizzled by row
-#define T_TILE_BYTES (128 * T_ROWB)
+// Workgroup of four waves (2 x 2); a wave owns FN x FM tiles of 16 x 16, so the
+// workgroup's tile is (32 FN) weight rows by (32 FM) activation rows.  K moves
+// through LDS two slabs at a time, double-buffered; 16-byte columns of a tile
+// row are XOR-swizzled by the row so that fragment reads do not collide.
+#define T_ROWB 128                     // LDS bytes per tile row: two slabs
 #define T_CHUNK_TILES (KC_SLABS / 2)   // K tiles (of two slabs) per chunk
 
+template <int FN, int FM>
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(elem_t* __restrict__ out, const elem_t* __restrict__ act,
                                                          const elem_t* __restrict__ w, int M, int N, int K,
                                                          int64_t lda, int64_t ldo, int out_vec_ok) {
-  __shared__ __attribute__((aligned(16))) unsigned char lds[2][2][T_TILE_BYTES];  // [buffer][0: w, 1: act]
+  constexpr int BN = 32 * FN, BM = 32 * FM;
+  constexpr int W_BYTES = BN * T_ROWB, A_BYTES = BM * T_ROWB, BUF_BYTES = W_BYTES + A_BYTES;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];   // [buffer][w tile, act tile]
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r16 = lane & 15, kg = lane >> 4;
   const int wn = wave & 1, wm = wave >> 1;
-  const int n_blk = blockIdx.x * T_BN, m_blk = blockIdx.y * T_BM;
+  const int n_blk = blockIdx.x * BN, m_blk = blockIdx.y * BM;
   const int nslabs = (K + VK_SLAB - 1) / VK_SLAB;
   const int ntiles = (nslabs + 1) / 2;
 
   // Global -> LDS mapping: thread loads 16 bytes at column c16 of rows lrow + 32*i.
   const int lrow = tid >> 3, c16 = tid & 7;
-  const elem_t* gw[4];
-  const elem_t* ga[4];
-  bool gw_ok[4], ga_ok[4];
+  const elem_t* gw[FN];
+  const elem_t* ga[FM];
+  bool gw_ok[FN], ga_ok[FM];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int n = n_blk + lrow + 32 * i, m = m_blk + lrow + 32 * i;
+  for (int i = 0; i < FN; ++i) {
+    const int n = n_blk + lrow + 32 * i;
     gw_ok[i] = n < N;
-    ga_ok[i] = m < M;
     gw[i] = w + (int64_t)(gw_ok[i] ? n : 0) * K + c16 * VK_VEC;
+  }
+#pragma unroll
+  for (int i = 0; i < FM; ++i) {
+    const int m = m_blk + lrow + 32 * i;
+    ga_ok[i] = m < M;
     ga[i] = act + (int64_t)(ga_ok[i] ? m : 0) * lda + c16 * VK_VEC;
   }
 
-  frag_t rw[4], ra[4];
+  frag_t rw[FN], ra[FM];
   auto gload = [&](int kt) {
     const int k = kt * 2 * VK_SLAB;
     const bool kok = k + c16 * VK_VEC < K;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      rw[i] = load_frag(gw[i] + k, gw_ok[i] && kok);
-      ra[i] = load_frag(ga[i] + k, ga_ok[i] && kok);
-    }
+    for (int i = 0; i < FN; ++i) rw[i] = load_frag(gw[i] + k, gw_ok[i] && kok);
+#pragma unroll
+    for (int i = 0; i < FM; ++i) ra[i] = load_frag(ga[i] + k, ga_ok[i] && kok);
   };
   auto lstore = [&](int buf) {
+    unsigned char* base = lds + buf * BUF_BYTES;
+    const int col = (c16 ^ (lrow & 7)) * 16;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int off = (lrow + 32 * i) * T_ROWB + ((c16 ^ (lrow & 7)) * 16);
-      *reinterpret_cast<frag_t*>(&lds[buf][0][off]) = rw[i];
-      *reinterpret_cast<frag_t*>(&lds[buf][1][off]) = ra[i];
+    for (int i = 0; i < FN; ++i) *reinterpret_cast<frag_t*>(base + (lrow + 32 * i) * T_ROWB + col) = rw[i];
+#pragma unroll
+    for (int i = 0; i < FM; ++i) *reinterpret_cast<frag_t*>(base + W_BYTES + (lrow + 32 * i) * T_ROWB + col) = ra[i];
+  };
+
+  f32x4 acc[FN][FM], total[FN][FM];
+#pragma unroll
+  for (int i = 0; i < FN; ++i)
+#pragma unroll
+    for (int j = 0; j < FM; ++j) {
+      acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+      total[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+
+  gload(0);
+  lstore(0);
+  __syncthreads();
+
+  for (int kt = 0; kt < ntiles; ++kt) {
+    const unsigned char* base = lds + (kt & 1) * BUF_BYTES;
+    if (kt + 1 < ntiles) gload(kt + 1);
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      frag_t wf[FN], af[FM];
+      const int col = ((s * 4 + kg) ^ (r16 & 7)) * 16;
+#pragma unroll
+      for (int i = 0; i < FN; ++i)
+        wf[i] = *reinterpret_cast<const frag_t*>(base + (wn * 16 * FN + i * 16 + r16) * T_ROWB + col);
+#pragma unroll
+      for (int j = 0; j < FM; ++j)
+        af[j] = *reinterpret_cast<const frag_t*>(base + W_BYTES + (wm * 16 * FM + j * 16 + r16) * T_ROWB + col);
+#pragma unroll
+      for (int i = 0; i < FN; ++i)
+#pragma unroll
+        for (int j = 0; j < FM; ++j) acc[i][j] = mma_slab(wf[i], af[j], acc[i][j]);
+    }
+    if ((kt + 1) % T_CHUNK_TILES == 0 || kt + 1 == ntiles) {
+#pragma unroll
+      for (int i = 0; i < FN; ++i)
+#pragma unroll
+        for (int j = 0; j < FM; ++j) {
+          total[i][j].x = total[i][j].x + acc[i][j].x;
+          total[i][j].y = total[i][j].y + acc[i][j].y;
+          total[i][j].z = total[i][j].z + acc[i][j].z;
+          total[i][j].w = total[i][j].w + acc[i][j].w;
+          acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+    }
+    if (kt + 1 < ntiles) lstore((kt & 1) ^ 1);
+    __syncthreads();
+  }
+
+#pragma unroll
+  for (int i = 0; i < FN; ++i)
+#pragma unroll
+    for (int j = 0; j < FM; ++j)
+      store_out4(out, ldo, m_blk + wm * 16 * FM + j * 16 + r16, n_blk + wn * 16 * FN + i * 16 + 4 * kg, M, N,
+                 total[i][j], out_vec_ok);
+}
+
+template <int FN, int FM>
+static int launch_tiled(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K, int64_t lda, int64_t ldo,
+                        int vec_ok, hipStream_t st) {
+  constexpr int BN = 32 * FN, BM = 32 * FM;
+  const size_t smem = 2 * (size_t)(BN + BM) * T_ROWB;
+  static bool configured = false;
+  if (!configured) {
+    if (smem > 48 * 1024)
+      (void)hipFuncSetAttribute((const void*)gemm_tiled_kernel<FN, FM>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)smem);
+    configured = true;
+  }
+  dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
+  VK_REQUIRE(grid.y <= 65535, "gemm: too many rows (%d)", M);
+  gemm_tiled_kernel<FN, FM><<<grid, 256, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok);
+  return vk_check_launch("gemm_tiled");
+}
+
+// --------------------------------------------------------------- pipelined
+// The tiled kernel for K a multiple of 64 bytes-per-row tiles (two slabs), with
+// what the other lacks to keep the MFMA units fed: tiles go from global memory
+// straight into LDS (global_load_lds_dwordx4, no registers in between) and S
+// stages are in flight, so a tile's latency is hidden behind the S-1 tiles
+// computed meanwhile.  One barrier per K tile.  Rows beyond N or M are clamped
+// (their results are dropped).  Same tile shape, swizzle and reduction order as
+// gemm_tiled_kernel<4, 4>.
+__device__ __forceinline__ void wait_vmcnt(int n) {
+  // s_waitcnt with only vmcnt set: vmcnt is bits [3:0] and [15:14]; expcnt and lgkmcnt left at their maxima.
+  switch (n) {
+    case 0: __builtin_amdgcn_s_waitcnt(0x0F70); break;
+    case 8: __builtin_amdgcn_s_waitcnt(0x0F78); break;
+    case 16: __builtin_amdgcn_s_waitcnt(0x4F70); break;
+    case 24: __builtin_amdgcn_s_waitcnt(0x4F78); break;
+    default: __builtin_amdgcn_s_waitcnt(0x0F70); break;
+  }
+}
+
+template <int S>
+__global__ __launch_bounds__(256) void gemm_pipe_kernel(elem_t* __restrict__ out, const elem_t* __restrict__ act,
+                                                        const elem_t* __restrict__ w, int M, int N, int K,
+                                                        int64_t lda, int64_t ldo, int out_vec_ok) {
+  constexpr int TILE_BYTES = 128 * T_ROWB, STAGE_BYTES = 2 * TILE_BYTES;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];   // [stage][w tile, act tile]
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r16 = lane & 15, kg = lane >> 4;
+  const int wn = wave & 1, wm = wave >> 1;
+  const int n_blk = blockIdx.x * 128, m_blk = blockIdx.y * 128;
+  const int ntiles = K / (2 * VK_SLAB);
+
+  // A wave-level load moves 8 rows x 128 bytes; lane i fills LDS slot i of the 1 KB block, which is
+  // row i/8, physical 16-byte column i%8, i.e. logical column (i%8) ^ (i/8).
+  const int lr = lane >> 3, lc = (lane & 7) ^ lr;
+  const elem_t* gw[4];
+  const elem_t* ga[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int row = (wave * 4 + j) * 8 + lr;
+    gw[j] = w + (int64_t)min(n_blk + row, N - 1) * K + lc * VK_VEC;
+    ga[j] = act + (int64_t)min(m_blk + row, M - 1) * lda + lc * VK_VEC;
+  }
+  auto issue = [&](int kt) {
+    unsigned char* base = lds + (kt % S) * STAGE_BYTES + (wave * 4) * 8 * T_ROWB;
+    const int k = kt * 2 * VK_SLAB;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      __builtin_amdgcn_global_load_lds(gw[j] + k, (__attribute__((address_space(3))) void*)(base + j * 8 * T_ROWB), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(ga[j] + k, (__attribute__((address_space(3))) void*)(base + TILE_BYTES + j * 8 * T_ROWB), 16, 0, 0);
     }
   };
 
@@ -281,21 +492,25 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(elem_t* __restrict__ ou
       total[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
-  gload(0);
-  lstore(0);
-  __syncthreads();
+#pragma unroll
+  for (int p = 0; p < S - 1; ++p)
+    if (p < ntiles) issue(p);
 
   for (int kt = 0; kt < ntiles; ++kt) {
-    const int buf = kt & 1;
-    if (kt + 1 < ntiles) gload(kt + 1);
+    // Tile kt has landed once at most the loads of the tiles after it are outstanding (8 per tile and wave).
+    const int later = min(S - 2, ntiles - 1 - kt);
+    wait_vmcnt(8 * later);
+    __syncthreads();       // every wave's part of tile kt is there; everyone is done with tile kt-1's buffer
+    if (kt + S - 1 < ntiles) issue(kt + S - 1);
+    const unsigned char* base = lds + (kt % S) * STAGE_BYTES;
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
       frag_t wf[4], af[4];
+      const int col = ((s * 4 + kg) ^ (r16 & 7)) * 16;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int col = ((s * 4 + kg) ^ (r16 & 7)) * 16;
-        wf[i] = *reinterpret_cast<const frag_t*>(&lds[buf][0][(wn * 64 + i * 16 + r16) * T_ROWB + col]);
-        af[i] = *reinterpret_cast<const frag_t*>(&lds[buf][1][(wm * 64 + i * 16 + r16) * T_ROWB + col]);
+        wf[i] = *reinterpret_cast<const frag_t*>(base + (wn * 64 + i * 16 + r16) * T_ROWB + col);
+        af[i] = *reinterpret_cast<const frag_t*>(base + TILE_BYTES + (wm * 64 + i * 16 + r16) * T_ROWB + col);
       }
 #pragma unroll
       for (int i = 0; i < 4; ++i)
@@ -314,8 +529,6 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(elem_t* __restrict__ ou
           acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
         }
     }
-    if (kt + 1 < ntiles) lstore(buf ^ 1);
-    __syncthreads();
   }
 
 #pragma unroll
@@ -326,11 +539,26 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(elem_t* __restrict__ ou
                  out_vec_ok);
 }
 
+template <int S>
+static int launch_pipe(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K, int64_t lda, int64_t ldo,
+                       int vec_ok, hipStream_t st) {
+  const size_t smem = (size_t)S * 2 * 128 * T_ROWB;
+  static bool configured = false;
+  if (!configured) {
+    (void)hipFuncSetAttribute((const void*)gemm_pipe_kernel<S>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    configured = true;
+  }
+  dim3 grid((N + 127) / 128, (M + 127) / 128);
+  VK_REQUIRE(grid.y <= 65535, "gemm: too many rows (%d)", M);
+  gemm_pipe_kernel<S><<<grid, 256, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok);
+  return vk_check_launch("gemm_pipe");
+}
+
 // ==================================================================== host
 extern "C" {
 
-// kernel: 0 = choose by M, 1 = skinny (M <= 64), 2 = tiled.  The result does not
-// depend on the choice.
+// kernel: 0 = choose by M, 1 = skinny (M <= 64), 2 = tiled (pipelined if K allows), 3 = tiled through
+// registers, 4..6 = pipelined with 2..4 stages (for measurements).  The result does not depend on the choice.
 int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K, int64_t lda, int64_t ldo,
             int kernel, hipStream_t st) {
   VK_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
@@ -339,7 +567,7 @@ int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K
              (long long)lda, VK_VEC);
   VK_REQUIRE(ldo >= N, "gemm: output row stride %lld is smaller than N=%d", (long long)ldo, N);
   VK_REQUIRE(((uintptr_t)act % 16) == 0 && ((uintptr_t)w % 16) == 0, "gemm: operands must be 16-byte aligned");
-  VK_REQUIRE(kernel >= 0 && kernel <= 2, "gemm: unknown kernel %d", kernel);
+  VK_REQUIRE(kernel >= 0 && kernel <= 6, "gemm: unknown kernel %d", kernel);
   if (M == 0) return 0;
   const int vec_ok = (ldo % 4 == 0) && ((uintptr_t)out % 16 == 0);
   if (kernel == 0) kernel = M <= 64 ? 1 : 2;
@@ -378,10 +606,38 @@ int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K
 #undef SK
     return vk_check_launch("gemm_skinny");
   }
-  dim3 grid((N + T_BN - 1) / T_BN, (M + T_BM - 1) / T_BM);
-  VK_REQUIRE(grid.y <= 65535, "gemm: too many rows (%d)", M);
-  gemm_tiled_kernel<<<grid, 256, 0, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok);
-  return vk_check_launch("gemm_tiled");
+  const bool k_whole = K % (2 * VK_SLAB) == 0;
+  if (kernel == 3) return launch_tiled<4, 4>(out, act, w, M, N, K, lda, ldo, vec_ok, st);
+  if (kernel == 4 && k_whole) return launch_pipe<2>(out, act, w, M, N, K, lda, ldo, vec_ok, st);
+  if (kernel == 5 && k_whole) return launch_pipe<3>(out, act, w, M, N, K, lda, ldo, vec_ok, st);
+  if (kernel == 6 && k_whole) return launch_pipe<4>(out, act, w, M, N, K, lda, ldo, vec_ok, st);
+  // Two stages of 32 KB leave room for two workgroups per compute unit, which hides more latency than a third stage.
+  if (k_whole) return launch_pipe<2>(out, act, w, M, N, K, lda, ldo, vec_ok, st);
+  return launch_tiled<4, 4>(out, act, w, M, N, K, lda, ldo, vec_ok, st);
+}
+
+// 1 if vk_gemm_swiglu takes these sizes (the caller otherwise runs vk_gemm and vk_swiglu, with the same result).
+int vk_gemm_swiglu_supported(int M, int I, int K) { return M >= 1 && M <= 16 && I > 0 && K % KC == 0 && K <= SK_WAVES * KC; }
+
+// out[M, I] = silu(act w_gate^T) * (act w_up^T), w = [gate rows; up rows] of shape [2I, K].
+int vk_gemm_swiglu(elem_t* out, const elem_t* act, const elem_t* w, int M, int I, int K, int64_t lda, int64_t ldo,
+                   hipStream_t st) {
+  VK_REQUIRE(vk_gemm_swiglu_supported(M, I, K), "gemm_swiglu: sizes M=%d I=%d K=%d are not supported", M, I, K);
+  VK_REQUIRE(lda >= K && lda % VK_VEC == 0 && ldo >= I, "gemm_swiglu: bad row strides");
+  VK_REQUIRE(((uintptr_t)act % 16) == 0 && ((uintptr_t)w % 16) == 0, "gemm_swiglu: operands must be 16-byte aligned");
+  static int resident = 0;
+  if (resident == 0) {
+    int dev = 0, cus = 0, per_cu = 0;
+    (void)hipGetDevice(&dev);
+    (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gemm_stream_swiglu_kernel<8>, 64 * SK_WAVES, 0);
+    resident = (cus > 0 ? cus : 256) * (per_cu > 0 ? per_cu : 1);
+  }
+  const int ntiles = (I + 15) / 16;
+  const int vec_ok = (ldo % 4 == 0) && ((uintptr_t)out % 16 == 0);
+  gemm_stream_swiglu_kernel<8><<<ntiles < resident ? ntiles : resident, 64 * SK_WAVES, 0, st>>>(out, act, w, M, I, K,
+                                                                                               lda, ldo, vec_ok);
+  return vk_check_launch("gemm_swiglu");
 }
 
 }  // extern "C"

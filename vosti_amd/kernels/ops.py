@@ -65,6 +65,8 @@ class Kernels:
         _sig(lib.vk_rope_tables, P, P, P, I, I, P)
         _sig(lib.vk_fill_random, P, L, c_uint64, I, F, F, P)
         _sig(lib.vk_gemm, P, P, P, I, I, I, L, L, I, P)
+        _sig(lib.vk_gemm_swiglu, P, P, P, I, I, I, L, L, P)
+        _sig(lib.vk_gemm_swiglu_supported, I, I, I)
         _sig(lib.vk_qkv_post, P, L, P, P, P, P, P, I, P, P, I, P, P, I, I, I, I, I, F, P)
         _sig(lib.vk_paged_attention, P, P, P, P, P, I, P, P, P, I, I, I, P, I, I, I, I, I, I, F, P)
         _sig(lib.vk_sample, P, P, P, P, P, I, I, L, P)
@@ -206,6 +208,25 @@ class Kernels:
         out = self.empty(M, N) if out is None else out
         self._elem(out, "out", M, N)
         self._call(self.lib.vk_gemm, out.data_ptr(), act.data_ptr(), w.data_ptr(), M, N, K, lda, N, kernel,
+                   self._stream())
+        return out
+
+    def gemm_swiglu(self, act: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
+        """silu(act @ w_gate.T) * (act @ w_up.T) with w_gate_up = [gate rows; up rows].
+
+        One launch where the sizes allow it, else the projection and the activation one after the
+        other; the result is the same bits either way."""
+        M, K = act.shape
+        N2, K2 = w_gate_up.shape
+        if K2 != K or N2 % 2:
+            raise KernelError(f"gemm_swiglu: activation [{M}, {K}] does not fit a gate/up weight [{N2}, {K2}]")
+        I = N2 // 2
+        if not (act.is_contiguous() and self.lib.vk_gemm_swiglu_supported(M, I, K)):
+            return self.swiglu(self.gemm(act, w_gate_up))
+        self._elem(act, "activation", M, K)
+        self._elem(w_gate_up, "weight", N2, K)
+        out = self.empty(M, I)
+        self._call(self.lib.vk_gemm_swiglu, out.data_ptr(), act.data_ptr(), w_gate_up.data_ptr(), M, I, K, K, I,
                    self._stream())
         return out
 

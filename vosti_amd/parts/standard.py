@@ -243,7 +243,7 @@ class SwiGLU(FeedForward):
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         k = self.kernels
-        return k.gemm(k.swiglu(k.gemm(x, self.w_gate_up)), self.w_down)
+        return k.gemm(k.gemm_swiglu(x, self.w_gate_up), self.w_down)
 
 
 @register_part("block", "prenorm")
