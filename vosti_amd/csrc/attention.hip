@@ -86,7 +86,7 @@ __device__ __forceinline__ void tile_partial(const RowCtx& c, const frag_t (&qf)
   const int64_t tile_page = one_page ? (int64_t)c.bt[kb >> lp] * c.page_stride : 0;
   const elem_t* kpage = c.kbase + tile_page;
   const elem_t* vpage = c.vbase + tile_page;
-  // ---- key fragments of the whole tile, then value fragments, all in flight together ----
+  // ---- key fragments of the whole tile, all in flight together ----
   constexpr int KSUB = S_PER_LANE / 4;    // 16-key MFMA sub-tiles per tile
   frag_t kf[KSUB][NQS];
 #pragma unroll
@@ -108,6 +108,22 @@ __device__ __forceinline__ void tile_partial(const RowCtx& c, const frag_t (&qf)
       }
     }
   }
+  // ---- scores S^T[key, row] = K Q^T ----
+  float sc[S_PER_LANE];
+#pragma unroll
+  for (int sub = 0; sub < KSUB; ++sub) {
+    f32x4 s4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < NQS; ++s)
+      if (s * VK_SLAB < d) s4 = mma_slab(kf[sub][s], qf[s], s4);
+    sc[4 * sub + 0] = s4.x;
+    sc[4 * sub + 1] = s4.y;
+    sc[4 * sub + 2] = s4.z;
+    sc[4 * sub + 3] = s4.w;
+  }
+  // ---- value fragments: requested once the key fragments' registers are free again, so that more
+  // waves fit a SIMD; their latency passes behind the softmax arithmetic and the other waves ----
+  __builtin_amdgcn_sched_barrier(0);
   frag_t vf[NDT][KEY_SLABS];
 #pragma unroll
   for (int dt = 0; dt < NDT; ++dt) {
@@ -121,19 +137,6 @@ __device__ __forceinline__ void tile_partial(const RowCtx& c, const frag_t (&qf)
         vf[dt][ks] = *reinterpret_cast<const frag_t*>(vrow);
       }
     }
-  }
-  // ---- scores S^T[key, row] = K Q^T ----
-  float sc[S_PER_LANE];
-#pragma unroll
-  for (int sub = 0; sub < KSUB; ++sub) {
-    f32x4 s4 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int s = 0; s < NQS; ++s)
-      if (s * VK_SLAB < d) s4 = mma_slab(kf[sub][s], qf[s], s4);
-    sc[4 * sub + 0] = s4.x;
-    sc[4 * sub + 1] = s4.y;
-    sc[4 * sub + 2] = s4.z;
-    sc[4 * sub + 3] = s4.w;
   }
   // ---- mask, maximum, probabilities ----
   bool vis[S_PER_LANE];

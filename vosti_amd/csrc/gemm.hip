@@ -570,7 +570,9 @@ int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K
   VK_REQUIRE(kernel >= 0 && kernel <= 6, "gemm: unknown kernel %d", kernel);
   if (M == 0) return 0;
   const int vec_ok = (ldo % 4 == 0) && ((uintptr_t)out % 16 == 0);
-  if (kernel == 0) kernel = M <= 64 ? 1 : 2;
+  // Measured on Qwen3-8B shapes: with more than 16 rows and many weight rows the pipelined kernel wins,
+  // with few weight rows it has too few workgroups and the streaming kernel does.
+  if (kernel == 0) kernel = (M <= 16 || (M <= 64 && N < 16384)) ? 1 : 2;
   if (kernel == 1) {
     VK_REQUIRE(M <= 64, "gemm: the skinny kernel takes at most 64 rows, got %d", M);
     const int mt = (M + 15) / 16;
