@@ -5,6 +5,7 @@ import pytest
 import torch
 
 import plain_qwen3 as plain
+from vosti_amd.kernels.ops import ATTN_ITEM_ROWS
 
 pytestmark = pytest.mark.gpu
 
@@ -265,7 +266,7 @@ def build_cache(kk, vv, P, n_pages, seed, dtype, poison=None):
     return kc, vc, table
 
 
-def run_attention(k, q_list, kk, vv, P, dtype, window=0, poison=None, decode_split=None, seed=0):
+def run_attention(k, q_list, kk, vv, P, dtype, window=0, poison=None, decode_split=None, seed=0, prompt_mode=0):
     n_pages = sum(-(-x.shape[0] // P) for x in kk) + 3
     kc, vc, table = build_cache(kk, vv, P, n_pages, seed, dtype, poison)
     q = torch.cat(q_list).cuda()
@@ -273,13 +274,13 @@ def run_attention(k, q_list, kk, vv, P, dtype, window=0, poison=None, decode_spl
     cu = torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32)
     k_len = torch.tensor([x.shape[0] for x in kk], dtype=torch.int32)
     out = torch.zeros_like(q)
-    pre = [(s, o) for s, n in enumerate(q_lens) if n > 1 for o in range(0, n, 16)]
+    pre = [(s, o) for s, n in enumerate(q_lens) if n > 1 for o in range(0, n, ATTN_ITEM_ROWS)]
     dec = [(s, 0) for s, n in enumerate(q_lens) if n == 1]
     d = q.shape[2]
     args = (q, kc.cuda(), vc.cuda(), table.cuda(), cu.cuda(), k_len.cuda())
     kw = dict(scale=d ** -0.5, window=window, max_k_len=int(k_len.max()), out=out)
     if pre:
-        k.paged_attention(*args, torch.tensor(pre, dtype=torch.int32).cuda(), mode=0, **kw)
+        k.paged_attention(*args, torch.tensor(pre, dtype=torch.int32).cuda(), mode=prompt_mode, **kw)
     if dec:
         items = torch.tensor(dec, dtype=torch.int32).cuda()
         nseg = -(-int(k_len.max()) // 256) + (1 if decode_split else 0)    # more segments than needed are harmless
@@ -310,6 +311,68 @@ def test_attention_against_plain(dtype, nq, nkv, d, P):
     # Poison changes nothing bitwise, nor does another page order or a wider segment grid.
     clean = run_attention(k, q_list, kk, vv, P, dtype, poison=None, decode_split=True, seed=5)
     assert torch.equal(clean, got)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,d,P,window", [(4, 1, 128, 64, 0), (6, 2, 64, 128, 0), (2, 2, 256, 64, 0), (3, 1, 128, 256, 0),
+                                               (4, 2, 128, 64, 150), (2, 1, 64, 64, 64), (8, 2, 64, 64, 333)])
+def test_attention_prompt_kernels_agree(dtype, nq, nkv, d, P, window):
+    """Prompt rows through the kernel that shares key tiles in LDS (these head and page sizes), through
+    the kernel for every shape, and as decoded tokens: the same bits, and the plain result.  Portions
+    of one to a few hundred rows after contexts that end inside tiles, segments and pages; NaN in every
+    unused page and tail."""
+    k = kern(dtype)
+    if dtype == torch.float32 and d == 256:
+        assert not k.lib.vk_attn_prefill_shares_tiles(d, P)
+    else:
+        assert k.lib.vk_attn_prefill_shares_tiles(d, P)
+    shapes = [(300, 300), (129, 641), (2, 64), (33, 289), (128, 128), (97, 1000), (31, 95), (64, 576)]
+    q_list, kk, vv = [], [], []
+    for i, (ql, kl) in enumerate(shapes):
+        q_list.append(rand((ql, nq, d), dtype, 10 + i))
+        kk.append(rand((kl, nkv, d), dtype, 30 + i))
+        vv.append(rand((kl, nkv, d), dtype, 50 + i))
+    got = run_attention(k, q_list, kk, vv, P, dtype, window=window, poison=float("nan"))
+    other = run_attention(k, q_list, kk, vv, P, dtype, window=window, poison=float("nan"), seed=3, prompt_mode=2)
+    assert torch.equal(got, other)
+    off = 0
+    for q, kx, vx in zip(q_list, kk, vv):
+        ref = plain.attention(q, kx, vx, d ** -0.5, dtype, window=window)
+        torch.testing.assert_close(got[off:off + q.shape[0]].float(), ref, **tol(dtype))
+        off += q.shape[0]
+    # The last rows of two sequences as decoded tokens.
+    for i in (1, 5):
+        q, kx, vx = q_list[i], kk[i], vv[i]
+        start = sum(x.shape[0] for x in q_list[:i])
+        one = run_attention(k, [q[-1:]], [kx], [vx], P, dtype, window=window)
+        assert torch.equal(one[0], got[start + q.shape[0] - 1])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_far_key_in_prompt_rows(dtype):
+    """A key that outweighs all others, seen from the rows of a late portion of a prompt: every row at
+    or after it must return its value, through the kernel that shares tiles and the other one.  Then
+    with a window that still holds the key for the first rows of the portion only."""
+    k = kern(dtype)
+    nq, nkv, d, P, L, n = 4, 2, 64, 64, 900, 200
+    for far in (0, 63, 64, 255, 256, 699, 700, 764, 899):
+        q = rand((n, nq, d), dtype, 1) * 0.1
+        kx, vx = rand((L, nkv, d), dtype, 2) * 0.1, rand((L, nkv, d), dtype, 3)
+        q[:, :, 0] = 40.0
+        kx[far, :, 0] = 40.0
+        want = vx[far].float().repeat_interleave(nq // nkv, dim=0)
+        for mode in (0, 2):
+            got = run_attention(k, [q], [kx], [vx], P, dtype, prompt_mode=mode)
+            first = max(0, far - (L - n))          # the first row of the portion that sees the key
+            torch.testing.assert_close(got[first:].float(), want.expand(n - first, -1, -1), **tol(dtype))
+            if first:
+                assert (got[:first].float() - want).abs().max() > 0.1
+        if far >= L - n:
+            continue
+        w = L - n - far + 50                        # rows 0..49 of the portion still see the key
+        got = run_attention(k, [q], [kx], [vx], P, dtype, window=w)
+        torch.testing.assert_close(got[:50].float(), want.expand(50, -1, -1), **tol(dtype))
+        assert (got[50:].float() - want).abs().max() > 0.1
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

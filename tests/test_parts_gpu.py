@@ -4,6 +4,7 @@ import torch
 
 import plain_qwen3 as plain
 from vosti_amd.config import PartSpec
+from vosti_amd.kernels.ops import ATTN_ITEM_ROWS
 
 pytestmark = pytest.mark.gpu
 DTYPES = [torch.float32, torch.bfloat16]
@@ -48,7 +49,7 @@ def step_context(kernels, starts, q_lens, page, pages_of, n_pages, window=0):
     for n in q_lens:
         cu.append(cu[-1] + n)
     k_len = [s + n for s, n in zip(starts, q_lens)]
-    pre = [(i, o) for i, n in enumerate(q_lens) if n > 1 for o in range(0, n, 16)]
+    pre = [(i, o) for i, n in enumerate(q_lens) if n > 1 for o in range(0, n, ATTN_ITEM_ROWS)]
     dec = [(i, 0) for i, n in enumerate(q_lens) if n == 1]
     scratch = torch.empty(1 << 20, device="cuda")
     return StepContext(kernels=kernels, num_tokens=sum(q_lens), num_seqs=len(q_lens), positions=i32(positions), cu_q=i32(cu),

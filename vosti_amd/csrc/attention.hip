@@ -38,6 +38,7 @@
 #define SEG_TILES 4
 #define KEY_SLABS (TILE_KEYS / VK_SLAB)   // key slabs per tile: 2 (bfloat16) or 4 (float)
 #define S_PER_LANE 16                     // scores per lane per tile
+#define ITEM_ROWS 128                     // rows of a prompt item
 
 struct AttnArgs {
   const elem_t* q;        // [T, nq, d]
@@ -68,6 +69,56 @@ struct RowCtx {
   bool row_ok;
   float scale_log2;
 };
+
+// Scores of one tile -> the tile's own statistics (m, l) of this lane's row and its probabilities,
+// rounded to the element type, as MFMA operands.  The row sees keys lo..pos.
+__device__ __forceinline__ void tile_softmax(float (&sc)[S_PER_LANE], int kb, int g, bool row_ok, int lo, int pos,
+                                             float scale_log2, float& m_t, float& l_t, frag_t (&pf)[KEY_SLABS]) {
+  bool vis[S_PER_LANE];
+  float tmax = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < S_PER_LANE; ++i) {
+    const int key = kb + (i / VK_VEC) * VK_SLAB + g * VK_VEC + (i % VK_VEC);
+    vis[i] = row_ok && key >= lo && key <= pos;
+    sc[i] = sc[i] * scale_log2;
+    tmax = fmaxf(tmax, vis[i] ? sc[i] : -INFINITY);
+  }
+  tmax = fmaxf(tmax, __shfl_xor(tmax, 16, VK_WAVE));
+  tmax = fmaxf(tmax, __shfl_xor(tmax, 32, VK_WAVE));
+  float psum = 0.f;
+  float pr[S_PER_LANE];
+#pragma unroll
+  for (int i = 0; i < S_PER_LANE; ++i) {
+    pr[i] = vis[i] ? fast_exp2(sc[i] - tmax) : 0.f;
+    psum = psum + pr[i];
+  }
+  psum = psum + __shfl_xor(psum, 16, VK_WAVE);
+  psum = psum + __shfl_xor(psum, 32, VK_WAVE);
+  m_t = tmax;
+  l_t = psum;
+#pragma unroll
+  for (int ks = 0; ks < KEY_SLABS; ++ks) {
+#ifdef VK_BF16
+#pragma unroll
+    for (int j = 0; j < 8; ++j) pf[ks][j] = (__bf16)pr[ks * 8 + j];
+#else
+    pf[ks] = f32x4{pr[ks * 4 + 0], pr[ks * 4 + 1], pr[ks * 4 + 2], pr[ks * 4 + 3]};
+#endif
+  }
+}
+
+// Keys outside [first, k_len) may lie in pages this sequence does not own
+// (never written, or given back once the window passed them): their values
+// are replaced by zero so that stale NaN or Inf cannot reach the sum.
+__device__ __forceinline__ void zero_unowned(frag_t (&vf)[KEY_SLABS], int kb, int g, int first, int k_len) {
+#pragma unroll
+  for (int ks = 0; ks < KEY_SLABS; ++ks) {
+    const int k0 = kb + ks * VK_SLAB + g * VK_VEC;
+#pragma unroll
+    for (int j = 0; j < VK_VEC; ++j)
+      if (k0 + j >= k_len || k0 + j < first) vf[ks][j] = (elem_t)0.f;
+  }
+}
 
 // One tile, reduced on its own: m, l and acc[NDT] of this lane's row.
 template <int NDT, int NQS>
@@ -138,56 +189,13 @@ __device__ __forceinline__ void tile_partial(const RowCtx& c, const frag_t (&qf)
       }
     }
   }
-  // ---- mask, maximum, probabilities ----
-  bool vis[S_PER_LANE];
-  float tmax = -INFINITY;
-#pragma unroll
-  for (int i = 0; i < S_PER_LANE; ++i) {
-    const int key = kb + (i / VK_VEC) * VK_SLAB + g * VK_VEC + (i % VK_VEC);
-    vis[i] = c.row_ok && key >= c.lo && key <= c.pos;
-    sc[i] = sc[i] * c.scale_log2;
-    tmax = fmaxf(tmax, vis[i] ? sc[i] : -INFINITY);
-  }
-  tmax = fmaxf(tmax, __shfl_xor(tmax, 16, VK_WAVE));
-  tmax = fmaxf(tmax, __shfl_xor(tmax, 32, VK_WAVE));
-  float psum = 0.f;
-  float pr[S_PER_LANE];
-#pragma unroll
-  for (int i = 0; i < S_PER_LANE; ++i) {
-    pr[i] = vis[i] ? fast_exp2(sc[i] - tmax) : 0.f;
-    psum = psum + pr[i];
-  }
-  psum = psum + __shfl_xor(psum, 16, VK_WAVE);
-  psum = psum + __shfl_xor(psum, 32, VK_WAVE);
-  m_t = tmax;
-  l_t = psum;
-  // ---- acc = V^T P^T from zero; P rounded to the element type ----
+  // ---- mask, maximum, probabilities; acc = V^T P^T from zero ----
   frag_t pf[KEY_SLABS];
-#pragma unroll
-  for (int ks = 0; ks < KEY_SLABS; ++ks) {
-#ifdef VK_BF16
-#pragma unroll
-    for (int j = 0; j < 8; ++j) pf[ks][j] = (__bf16)pr[ks * 8 + j];
-#else
-    pf[ks] = f32x4{pr[ks * 4 + 0], pr[ks * 4 + 1], pr[ks * 4 + 2], pr[ks * 4 + 3]};
-#endif
-  }
-  // Keys outside [wave_lo, k_len) may lie in pages this sequence does not own
-  // (never written, or given back once the window passed them): their values
-  // are replaced by zero so that stale NaN or Inf cannot reach the sum.
+  tile_softmax(sc, kb, g, c.row_ok, c.lo, c.pos, c.scale_log2, m_t, l_t, pf);
   if (kb + TILE_KEYS > c.k_len || kb < c.wave_lo) {
 #pragma unroll
-    for (int dt = 0; dt < NDT; ++dt) {
-      if (dt * 16 < d) {
-#pragma unroll
-        for (int ks = 0; ks < KEY_SLABS; ++ks) {
-          const int k0 = kb + ks * VK_SLAB + g * VK_VEC;
-#pragma unroll
-          for (int j = 0; j < VK_VEC; ++j)
-            if (k0 + j >= c.k_len || k0 + j < c.wave_lo) vf[dt][ks][j] = (elem_t)0.f;
-        }
-      }
-    }
+    for (int dt = 0; dt < NDT; ++dt)
+      if (dt * 16 < d) zero_unowned(vf[dt], kb, g, c.wave_lo, c.k_len);
   }
 #pragma unroll
   for (int dt = 0; dt < NDT; ++dt) {
@@ -246,9 +254,11 @@ __device__ __forceinline__ void init_ctx(RowCtx& c, const AttnArgs& a, int seq, 
   c.scale_log2 = a.scale_log2;
 }
 
-// Prompt portions: an item is up to 16 consecutive rows of one sequence.  A
-// workgroup has one wave per q head of a kv head (up to 4), so that the waves
-// of a group read the same keys and values at about the same time.
+// Prompt portions, the kernel for every head size and page size: an item is up
+// to ITEM_ROWS consecutive rows of one sequence, a workgroup takes 16 of them.
+// It has one wave per q head of a kv head (up to 4), so that the waves of a
+// group read the same keys and values, straight from global memory, at about
+// the same time.
 template <int DPAD>
 __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a, int heads_per_wg) {
   constexpr int NDT = DPAD / 16, NQS = DPAD / VK_SLAB;
@@ -259,8 +269,11 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a, int heads
   const int hg = (blockIdx.y - kvh * groups_per_kv) * heads_per_wg + wave;
   if (hg >= G) return;
   const int head = kvh * G + hg;
-  const int seq = a.items[2 * blockIdx.x], q_off = a.items[2 * blockIdx.x + 1];
+  const int item = blockIdx.x / (ITEM_ROWS / 16);
+  const int seq = a.items[2 * item];
+  const int q_off = a.items[2 * item + 1] + (blockIdx.x % (ITEM_ROWS / 16)) * 16;
   const int q_begin = a.cu_q[seq], q_len = a.cu_q[seq + 1] - q_begin;
+  if (q_off >= q_len) return;
   const int k_len = a.k_len[seq];
   RowCtx c;
   init_ctx(c, a, seq, kvh, k_len);
@@ -304,6 +317,221 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a, int heads
       if (dt * 16 < a.d) {
         const float o[4] = {ACC[dt].x * inv, ACC[dt].y * inv, ACC[dt].z * inv, ACC[dt].w * inv};
         elem_t* p = orow + dt * 16 + 4 * c.g;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) p[i] = from_f32<elem_t>(o[i]);
+      }
+    }
+  }
+}
+
+// Prompt portions, the fast kernel: head sizes 64, 128, 256 with pages of at
+// least a tile.  A workgroup is one q head and one item; wave w has the rows
+// 32w .. 32w+31 as two 16-row tiles.  Every key tile goes from global memory
+// straight into LDS once (global_load_lds_dwordx4, two buffers: the next tile
+// lands while this one is used) and is read from there by all waves; a key or
+// value fragment read from LDS serves both row tiles of a wave.  The
+// arithmetic per row is tile_partial's and fold's, operation for operation.
+//
+// LDS holds the key tile as [64 keys][d] and the value tile as [d][64 keys],
+// in 16-byte columns that are XOR-swizzled by row so that the 16 lanes of a
+// fragment read hit different banks.  A wave-level load fills 1 KB of LDS in
+// lane order, so the swizzle is applied to the global address a lane reads.
+__device__ __forceinline__ void wait_vm_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }   // vmcnt(0) only
+// 16 bytes per lane from global memory into LDS at dst + 16 * lane (dst is the same for the wave).
+__device__ __forceinline__ void load_to_lds16(const elem_t* src, unsigned char* dst) {
+  __builtin_amdgcn_global_load_lds(src, (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+}
+
+#ifdef VK_BF16
+// MFMA row r16 of key sub-tile `sub` (see tile_partial) and the swizzle of a key row.
+__device__ __forceinline__ int key_row_of(int sub, int r16) { return (sub >> 1) * VK_SLAB + 8 * (r16 >> 2) + 4 * (sub & 1) + (r16 & 3); }
+__device__ __forceinline__ int key_swz(int row) { return (((row >> 3) & 3) << 2) | (row & 3); }
+__device__ __forceinline__ int val_swz(int row) { return (row >> 1) & 7; }    // rows of 128 bytes
+#else
+__device__ __forceinline__ int key_row_of(int sub, int r16) { return sub * VK_SLAB + r16; }
+__device__ __forceinline__ int key_swz(int row) { return row & 15; }
+__device__ __forceinline__ int val_swz(int row) { return row & 15; }          // rows of 256 bytes
+#endif
+
+template <int DPAD>
+__global__ __launch_bounds__(256) void attn_prefill_lds_kernel(AttnArgs a, int n_items) {
+  constexpr int NDT = DPAD / 16, NQS = DPAD / VK_SLAB;
+  constexpr int EB = (int)sizeof(elem_t);
+  constexpr int KRB = DPAD * EB, CK = KRB / 16;          // key row: bytes, 16-byte columns
+  constexpr int VRB = TILE_KEYS * EB, CV = VRB / 16;     // value row (one d index, 64 keys)
+  constexpr int KT_BYTES = TILE_KEYS * KRB, STAGE = 2 * KT_BYTES;   // value tile: DPAD * VRB, the same
+  constexpr int NI = CK / 4;                             // wave-level loads per wave for keys; as many for values
+  constexpr int KMASK = CK >= 16 ? 15 : CK - 1;
+  static_assert(CK % 4 == 0 && CK >= 8, "head size too small for this kernel");
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];   // [2][key tile, value tile]
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r16 = lane & 15, g = lane >> 4;
+  // Workgroups that run together on a chip quarter (every 8th index) get the q heads of the same
+  // item, which share keys; long items first.
+  const int total = n_items * a.nq;
+  const int lin = blockIdx.x;
+  const int v = total % 8 == 0 ? (lin & 7) * (total >> 3) + (lin >> 3) : lin;
+  const int item = n_items - 1 - v / a.nq, head = v % a.nq;
+  const int kvh = head / (a.nq / a.nkv);
+  const int seq = a.items[2 * item], q_off0 = a.items[2 * item + 1];
+  const int q_begin = a.cu_q[seq], q_len = a.cu_q[seq + 1] - q_begin;
+  const int k_len = a.k_len[seq];
+  const int rows_item = min(ITEM_ROWS, q_len - q_off0);
+  const int pos_item = k_len - q_len + q_off0;           // position of the item's first row
+  const int item_lo = a.window > 0 ? max(0, pos_item - a.window + 1) : 0;
+  const int tile_lo = item_lo / TILE_KEYS, tile_hi = (pos_item + rows_item - 1) / TILE_KEYS;
+
+  // ---- this wave's rows ----
+  const int rows_wave = min(32, rows_item - 32 * wave);  // <= 0: the wave only helps to load
+  const int pos_wave = pos_item + 32 * wave;
+  const int wave_lo = a.window > 0 ? max(0, pos_wave - a.window + 1) : 0;
+  const int wtile_lo = wave_lo / TILE_KEYS, wtile_hi = rows_wave > 0 ? (pos_wave + rows_wave - 1) / TILE_KEYS : -1;
+  bool row_ok[2];
+  int pos[2], lo[2], tok[2];
+  frag_t qf[2][NQS];
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt) {
+    row_ok[qt] = 16 * qt + r16 < rows_wave;
+    pos[qt] = pos_wave + 16 * qt + r16;
+    lo[qt] = a.window > 0 ? max(0, pos[qt] - a.window + 1) : 0;
+    tok[qt] = q_begin + q_off0 + 32 * wave + 16 * qt + r16;
+    load_q<NQS>(a, tok[qt], head, row_ok[qt], g, qf[qt]);
+  }
+
+  // ---- what this lane fetches of every tile ----
+  const int64_t page_elems = (int64_t)a.P * a.d;
+  const elem_t* kbase = a.kc + (int64_t)kvh * page_elems;
+  const elem_t* vbase = a.vc + (int64_t)kvh * page_elems;
+  const int64_t page_stride = (int64_t)a.nkv * page_elems;
+  const int32_t* bt = a.block_table + (int64_t)seq * a.bt_stride;
+  const int lp = __builtin_ctz(a.P);
+  int koff[NI], voff[NI];       // element offsets from the tile's first key (keys) or from its page row 0 (values)
+#pragma unroll
+  for (int j = 0; j < NI; ++j) {
+    const int instr = wave + 4 * j;                        // 1 KB of the tile each
+    const int krow = instr * (1024 / KRB) + lane / CK;     // key within the tile
+    const int kcol = (lane % CK) ^ (key_swz(krow) & KMASK);
+    koff[j] = krow * DPAD + kcol * VK_VEC;
+    const int vrow = instr * (1024 / VRB) + lane / CV;     // index along d
+    const int vcol = (lane % CV) ^ val_swz(vrow);
+    voff[j] = vrow * a.P + vcol * VK_VEC;
+  }
+  auto issue = [&](int t, int stage) {
+    const int kb = t * TILE_KEYS;
+    const int64_t page = (int64_t)bt[kb >> lp] * page_stride;
+    const int in_page = kb & (a.P - 1);
+    const elem_t* kt = kbase + page + (int64_t)in_page * DPAD;
+    const elem_t* vt = vbase + page + in_page;
+    unsigned char* dst = lds + stage * STAGE + wave * 1024;
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      load_to_lds16(kt + koff[j], dst + j * 4096);
+      load_to_lds16(vt + voff[j], dst + KT_BYTES + j * 4096);
+    }
+  };
+
+  float M[2], L[2], Ms[2], Ls[2];
+  f32x4 ACC[2][NDT], As[2][NDT];
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt) {
+    M[qt] = Ms[qt] = -INFINITY;
+    L[qt] = Ls[qt] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) ACC[qt][dt] = As[qt][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  issue(tile_lo, 0);
+  for (int t = tile_lo; t <= tile_hi; ++t) {
+    const int stage = (t - tile_lo) & 1;
+    wait_vm_loads();
+    __syncthreads();      // tile t is in LDS; every wave is done with the other buffer
+    if (t < tile_hi) issue(t + 1, stage ^ 1);
+    if (t >= wtile_lo && t <= wtile_hi) {
+      const int kb = t * TILE_KEYS;
+      const unsigned char* kl = lds + stage * STAGE;
+      const unsigned char* vl = kl + KT_BYTES;
+      // ---- scores of both row tiles ----
+      float sc[2][S_PER_LANE];
+#pragma unroll
+      for (int sub = 0; sub < S_PER_LANE / 4; ++sub) {
+        const int krow = key_row_of(sub, r16);
+        const unsigned char* kr = kl + krow * KRB;
+        const int sw = key_swz(krow) & KMASK;
+        frag_t kf[NQS];
+#pragma unroll
+        for (int s = 0; s < NQS; ++s) kf[s] = *reinterpret_cast<const frag_t*>(kr + (((s * 4 + g) ^ sw) << 4));
+#pragma unroll
+        for (int qt = 0; qt < 2; ++qt) {
+          f32x4 s4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int s = 0; s < NQS; ++s) s4 = mma_slab(kf[s], qf[qt][s], s4);
+          sc[qt][4 * sub + 0] = s4.x;
+          sc[qt][4 * sub + 1] = s4.y;
+          sc[qt][4 * sub + 2] = s4.z;
+          sc[qt][4 * sub + 3] = s4.w;
+        }
+      }
+      // ---- each row's own statistics of this tile, and how they fold into the segment's ----
+      frag_t pf[2][KEY_SLABS];
+      float ca[2], cb[2];
+      bool some[2];
+#pragma unroll
+      for (int qt = 0; qt < 2; ++qt) {
+        float m_t, l_t, Mn;
+        tile_softmax(sc[qt], kb, g, row_ok[qt], lo[qt], pos[qt], a.scale_log2, m_t, l_t, pf[qt]);
+        some[qt] = m_t > -INFINITY;
+        fold_scales(Ms[qt], m_t, Mn, ca[qt], cb[qt]);
+        if (some[qt]) {
+          Ls[qt] = fold1(Ls[qt], l_t, ca[qt], cb[qt]);
+          Ms[qt] = Mn;
+        }
+      }
+      // ---- P V from zero, folded into the segment's sum column block by column block ----
+      const bool edge = kb + TILE_KEYS > k_len || kb < wave_lo;
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt) {
+        const int vrow = dt * 16 + r16;
+        const unsigned char* vr = vl + vrow * VRB;
+        const int sw = val_swz(vrow);
+        frag_t vf[KEY_SLABS];
+#pragma unroll
+        for (int ks = 0; ks < KEY_SLABS; ++ks) vf[ks] = *reinterpret_cast<const frag_t*>(vr + (((ks * 4 + g) ^ sw) << 4));
+        if (edge) zero_unowned(vf, kb, g, wave_lo, k_len);
+#pragma unroll
+        for (int qt = 0; qt < 2; ++qt) {
+          f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int ks = 0; ks < KEY_SLABS; ++ks) acc = mma_slab(vf[ks], pf[qt][ks], acc);
+          if (some[qt]) {
+            As[qt][dt].x = fold1(As[qt][dt].x, acc.x, ca[qt], cb[qt]);
+            As[qt][dt].y = fold1(As[qt][dt].y, acc.y, ca[qt], cb[qt]);
+            As[qt][dt].z = fold1(As[qt][dt].z, acc.z, ca[qt], cb[qt]);
+            As[qt][dt].w = fold1(As[qt][dt].w, acc.w, ca[qt], cb[qt]);
+          }
+        }
+      }
+    }
+    if ((t + 1) % SEG_TILES == 0 || t == tile_hi) {        // the segment is complete
+#pragma unroll
+      for (int qt = 0; qt < 2; ++qt) {
+        fold<NDT>(M[qt], L[qt], ACC[qt], Ms[qt], Ls[qt], As[qt]);
+        Ms[qt] = -INFINITY;
+        Ls[qt] = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt) As[qt][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+      }
+    }
+  }
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt) {
+    if (row_ok[qt]) {
+      const float inv = L[qt] > 0.f ? 1.0f / L[qt] : 0.f;
+      elem_t* orow = a.out + ((int64_t)tok[qt] * a.nq + head) * a.d;
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt) {
+        const float o[4] = {ACC[qt][dt].x * inv, ACC[qt][dt].y * inv, ACC[qt][dt].z * inv, ACC[qt][dt].w * inv};
+        elem_t* p = orow + dt * 16 + 4 * g;
 #pragma unroll
         for (int i = 0; i < 4; ++i) p[i] = from_f32<elem_t>(o[i]);
       }
@@ -454,11 +682,20 @@ int64_t vk_attn_scratch_floats(int tokens, int nq, int d, int nseg) {
 
 int vk_attn_segment_keys(void) { return TILE_KEYS * SEG_TILES; }
 
-// items: n_items pairs (sequence, first row).  mode 0: each item is up to 16
-// consecutive rows of the sequence's q_len new tokens.  mode 1: each item is one
-// token; the keys are split by segment over nseg workgroups (nseg must cover
-// the longest sequence; scratch must hold vk_attn_scratch_floats(T, ...)) and
-// folded by a second kernel.  The result is the same in both modes.
+int vk_attn_item_rows(void) { return ITEM_ROWS; }
+
+// 1 if prompt rows of this shape go through the kernel that shares key tiles in LDS.
+int vk_attn_prefill_shares_tiles(int d, int P) {
+  return (d == 64 || d == 128 || d == 256) && P >= TILE_KEYS && 4 * TILE_KEYS * d * (int)sizeof(elem_t) <= 128 * 1024;
+}
+
+// items: n_items pairs (sequence, first row).  mode 0 and 2: each item is up to
+// vk_attn_item_rows() consecutive rows of the sequence's q_len new tokens
+// (mode 2 forces the kernel that takes every shape; the result is the same).
+// mode 1: each item is one token; the keys are split by segment over nseg
+// workgroups (nseg must cover the longest sequence; scratch must hold
+// vk_attn_scratch_floats(T, ...)) and folded by a second kernel.  The result
+// is the same in all modes.
 int vk_paged_attention(elem_t* out, const elem_t* q, const elem_t* kc, const elem_t* vc,
                        const int32_t* block_table, int bt_stride, const int32_t* cu_q, const int32_t* k_len,
                        const int32_t* items, int n_items, int mode, int nseg, float* scratch, int total_tokens,
@@ -467,7 +704,7 @@ int vk_paged_attention(elem_t* out, const elem_t* q, const elem_t* kc, const ele
   VK_REQUIRE(d >= 16 && d <= 256 && d % 16 == 0, "attention: head size %d must be a multiple of 16 in 16..256", d);
   VK_REQUIRE(P >= 8 && (P & (P - 1)) == 0, "attention: page size %d must be a power of two >= 8", P);
   VK_REQUIRE(window >= 0, "attention: window %d must not be negative", window);
-  VK_REQUIRE(mode == 0 || mode == 1, "attention: unknown mode %d", mode);
+  VK_REQUIRE(mode >= 0 && mode <= 2, "attention: unknown mode %d", mode);
   if (n_items <= 0) return 0;
   AttnArgs a;
   a.q = q; a.out = out; a.kc = kc; a.vc = vc; a.block_table = block_table; a.cu_q = cu_q; a.k_len = k_len;
@@ -475,9 +712,29 @@ int vk_paged_attention(elem_t* out, const elem_t* q, const elem_t* kc, const ele
   a.nseg = nseg; a.scale_log2 = scale * 1.4426950408889634f;
   a.part_ml = nullptr; a.part_acc = nullptr;
   const int G = nq / nkv;
-  if (mode == 0) {
+  if (mode == 0 && vk_attn_prefill_shares_tiles(d, P)) {
+    VK_REQUIRE((int64_t)n_items * nq < (1ll << 31), "attention: too many prompt items");
+    const size_t smem = (size_t)4 * TILE_KEYS * d * sizeof(elem_t);
+#define PREFILL_LDS(DP)                                                                              \
+  do {                                                                                               \
+    static bool raised = false;                                                                      \
+    if (!raised) {                                                                                   \
+      (void)hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<DP>,                            \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);             \
+      raised = true;                                                                                 \
+    }                                                                                                \
+    attn_prefill_lds_kernel<DP><<<n_items * nq, 256, smem, st>>>(a, n_items);                        \
+  } while (0)
+    if (d == 64) PREFILL_LDS(64);
+    else if (d == 128) PREFILL_LDS(128);
+    else PREFILL_LDS(256);
+#undef PREFILL_LDS
+    return vk_check_launch("attention (prompt rows, shared tiles)");
+  }
+  if (mode != 1) {
     const int hpw = G < 4 ? G : 4;
-    const dim3 grid(n_items, nkv * ((G + hpw - 1) / hpw));
+    VK_REQUIRE((int64_t)n_items * (ITEM_ROWS / 16) < (1ll << 31), "attention: too many prompt items");
+    const dim3 grid(n_items * (ITEM_ROWS / 16), nkv * ((G + hpw - 1) / hpw));
     VK_REQUIRE(grid.y <= 65535, "attention: too many heads");
     if (d <= 64) attn_prefill_kernel<64><<<grid, 64 * hpw, 0, st>>>(a, hpw);
     else if (d <= 128) attn_prefill_kernel<128><<<grid, 64 * hpw, 0, st>>>(a, hpw);

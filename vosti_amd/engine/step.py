@@ -22,10 +22,9 @@ import numpy as np
 import torch
 
 from ..cache import CachePool
-from ..kernels.ops import SEGMENT_KEYS
+from ..kernels.ops import ATTN_ITEM_ROWS, SEGMENT_KEYS
 from ..parts.base import GroupTables, StepContext
 
-ROW_TILE = 16          # rows of one attention work item
 WIDTH_BUCKET = 8       # captured block tables grow in steps of this many pages
 
 
@@ -137,7 +136,7 @@ class ModelRunner:
             if n == 1:
                 decode_items.append((s, 0))
             else:
-                prefill_items.extend((s, off) for off in range(0, n, ROW_TILE))
+                prefill_items.extend((s, off) for off in range(0, n, ATTN_ITEM_ROWS))
         parts: list[np.ndarray] = [ids.astype(np.int32), positions, cu_q, k_len, state_slots,
                                    np.asarray(want, dtype=np.int32),
                                    np.asarray(prefill_items, dtype=np.int32).reshape(-1, 2),

@@ -15,8 +15,9 @@ import torch
 
 from . import build
 
-ABI_VERSION = 9
+ABI_VERSION = 10
 SEGMENT_KEYS = 256
+ATTN_ITEM_ROWS = 128      # rows of one prompt item of paged_attention
 
 _DTYPES = {"bf16": torch.bfloat16, "f32": torch.float32}
 _NAMES = {torch.bfloat16: "bf16", torch.float32: "f32", "bfloat16": "bf16", "float32": "f32", "bf16": "bf16",
@@ -76,6 +77,8 @@ class Kernels:
         lib.vk_attn_scratch_floats.restype = c_int64
         lib.vk_attn_segment_keys.restype = c_int
         assert lib.vk_attn_segment_keys() == SEGMENT_KEYS
+        lib.vk_attn_item_rows.restype = c_int
+        assert lib.vk_attn_item_rows() == ATTN_ITEM_ROWS
         self.lib = lib
 
     # ------------------------------------------------------------ helpers
@@ -283,7 +286,10 @@ class Kernels:
                         out: torch.Tensor | None = None) -> torch.Tensor:
         """Attention of the rows named by ``items`` over the paged cache (see attention.hip).
 
-        ``max_k_len`` is the host's bound on k_len; the block table must cover it."""
+        items [n, 2] = (sequence, first row).  mode 0: an item is up to ATTN_ITEM_ROWS consecutive new
+        rows of its sequence; mode 2: the same through the kernel that takes every shape (same bits);
+        mode 1: an item is a single decoded token.  ``max_k_len`` is the host's bound on k_len; the
+        block table must cover it."""
         T, nq, d = q.shape
         pages, nkv, P, d2 = k_cache.shape
         S, W = block_table.shape

@@ -108,7 +108,7 @@ class StepContext:
     k_len: torch.Tensor          # [S]: keys of each sequence once this step's tokens are stored
     state_slots: torch.Tensor    # [S]: the state slot of each sequence
     groups: list[GroupTables]
-    prefill_items: torch.Tensor  # [n, 2]: (sequence, first row) of 16-row tiles of multi-token rows
+    prefill_items: torch.Tensor  # [n, 2]: (sequence, first row) of blocks of ATTN_ITEM_ROWS rows of multi-token sequences
     decode_items: torch.Tensor   # [n, 2]: single-token sequences
     max_k_len: int               # host copies, for launch geometry
     max_decode_k_len: int
