@@ -19,7 +19,7 @@
 //            empty (m = -inf).
 //   segment  4 tiles (256 keys).  Its non-empty tiles are folded, ascending,
 //            into a state that starts empty:
-//              M' = max(M, m); ACC' = ACC * 2^(M - M') + acc * 2^(m - M'); L' likewise.
+//              M' = max(M, m); ACC' = fma(acc, 2^(m - M'), ACC * 2^(M - M')); L' likewise.
 //   total    the non-empty segments are folded, ascending, the same way.
 // The prompt kernel folds in registers as it walks the tiles.  The decode
 // kernel gives every tile of a segment to a wave of its own, folds the four in
@@ -30,6 +30,8 @@
 // so that both MFMA operands of both products are 16-byte loads from global
 // memory: S^T = K Q^T and O^T = V^T P^T, which keeps a query row in one lane
 // column from scores to output.
+#include <type_traits>
+
 #include "common.h"
 #include "mma.h"
 #include "vec.h"
@@ -71,30 +73,48 @@ struct RowCtx {
 };
 
 // Scores of one tile -> the tile's own statistics (m, l) of this lane's row and its probabilities,
-// rounded to the element type, as MFMA operands.  The row sees keys lo..pos.
+// rounded to the element type, as MFMA operands.  The row sees keys lo..pos.  m is the largest
+// visible score times scale_log2 (> 0), a probability is 2^(score * scale_log2 - m) with the product
+// and the difference rounded once (a fused multiply-add).  `full` (the same for the whole wave) says
+// that every row of the wave sees every key of the tile: then the masks are left out, which changes
+// no bit.
 __device__ __forceinline__ void tile_softmax(float (&sc)[S_PER_LANE], int kb, int g, bool row_ok, int lo, int pos,
-                                             float scale_log2, float& m_t, float& l_t, frag_t (&pf)[KEY_SLABS]) {
-  bool vis[S_PER_LANE];
-  float tmax = -INFINITY;
-#pragma unroll
-  for (int i = 0; i < S_PER_LANE; ++i) {
-    const int key = kb + (i / VK_VEC) * VK_SLAB + g * VK_VEC + (i % VK_VEC);
-    vis[i] = row_ok && key >= lo && key <= pos;
-    sc[i] = sc[i] * scale_log2;
-    tmax = fmaxf(tmax, vis[i] ? sc[i] : -INFINITY);
-  }
-  tmax = fmaxf(tmax, __shfl_xor(tmax, 16, VK_WAVE));
-  tmax = fmaxf(tmax, __shfl_xor(tmax, 32, VK_WAVE));
-  float psum = 0.f;
+                                             float scale_log2, bool full, float& m_t, float& l_t,
+                                             frag_t (&pf)[KEY_SLABS]) {
   float pr[S_PER_LANE];
+  float psum = 0.f;
+  if (full) {
+    float tmax = sc[0];
 #pragma unroll
-  for (int i = 0; i < S_PER_LANE; ++i) {
-    pr[i] = vis[i] ? fast_exp2(sc[i] - tmax) : 0.f;
-    psum = psum + pr[i];
+    for (int i = 1; i < S_PER_LANE; ++i) tmax = fmaxf(tmax, sc[i]);
+    tmax = fmaxf(tmax, lane_xor16(tmax));
+    tmax = fmaxf(tmax, lane_xor32(tmax));
+    m_t = tmax * scale_log2;
+#pragma unroll
+    for (int i = 0; i < S_PER_LANE; ++i) {
+      pr[i] = fast_exp2(__builtin_fmaf(sc[i], scale_log2, -m_t));
+      psum = psum + pr[i];
+    }
+  } else {
+    bool vis[S_PER_LANE];
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < S_PER_LANE; ++i) {
+      const int key = kb + (i / VK_VEC) * VK_SLAB + g * VK_VEC + (i % VK_VEC);
+      vis[i] = row_ok && key >= lo && key <= pos;
+      tmax = fmaxf(tmax, vis[i] ? sc[i] : -INFINITY);
+    }
+    tmax = fmaxf(tmax, lane_xor16(tmax));
+    tmax = fmaxf(tmax, lane_xor32(tmax));
+    m_t = tmax * scale_log2;
+#pragma unroll
+    for (int i = 0; i < S_PER_LANE; ++i) {
+      pr[i] = vis[i] ? fast_exp2(__builtin_fmaf(sc[i], scale_log2, -m_t)) : 0.f;
+      psum = psum + pr[i];
+    }
   }
-  psum = psum + __shfl_xor(psum, 16, VK_WAVE);
-  psum = psum + __shfl_xor(psum, 32, VK_WAVE);
-  m_t = tmax;
+  psum = psum + lane_xor16(psum);
+  psum = psum + lane_xor32(psum);
   l_t = psum;
 #pragma unroll
   for (int ks = 0; ks < KEY_SLABS; ++ks) {
@@ -191,7 +211,7 @@ __device__ __forceinline__ void tile_partial(const RowCtx& c, const frag_t (&qf)
   }
   // ---- mask, maximum, probabilities; acc = V^T P^T from zero ----
   frag_t pf[KEY_SLABS];
-  tile_softmax(sc, kb, g, c.row_ok, c.lo, c.pos, c.scale_log2, m_t, l_t, pf);
+  tile_softmax(sc, kb, g, c.row_ok, c.lo, c.pos, c.scale_log2, false, m_t, l_t, pf);
   if (kb + TILE_KEYS > c.k_len || kb < c.wave_lo) {
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt)
@@ -213,7 +233,7 @@ __device__ __forceinline__ void fold_scales(float M, float m, float& Mn, float& 
   ca = fast_exp2(M - Mn);
   cb = fast_exp2(m - Mn);
 }
-__device__ __forceinline__ float fold1(float A, float a, float ca, float cb) { return A * ca + a * cb; }
+__device__ __forceinline__ float fold1(float A, float a, float ca, float cb) { return __builtin_fmaf(a, cb, A * ca); }
 
 template <int NDT>
 __device__ __forceinline__ void fold(float& M, float& L, f32x4 (&ACC)[NDT], float m, float l, const f32x4 (&acc)[NDT]) {
@@ -325,8 +345,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a, int heads
 }
 
 // Prompt portions, the fast kernel: head sizes 64, 128, 256 with pages of at
-// least a tile.  A workgroup is one q head and one item; wave w has the rows
-// 32w .. 32w+31 as two 16-row tiles.  Every key tile goes from global memory
+// least a tile.  A workgroup is one q head and one item; each of its waves has
+// QT 16-row tiles of the item's rows.  Every key tile goes from global memory
 // straight into LDS once (global_load_lds_dwordx4, two buffers: the next tile
 // lands while this one is used) and is read from there by all waves; a key or
 // value fragment read from LDS serves both row tiles of a wave.  The
@@ -353,49 +373,64 @@ __device__ __forceinline__ int key_swz(int row) { return row & 15; }
 __device__ __forceinline__ int val_swz(int row) { return row & 15; }          // rows of 256 bytes
 #endif
 
-template <int DPAD>
-__global__ __launch_bounds__(256) void attn_prefill_lds_kernel(AttnArgs a, int n_items) {
+template <int DPAD, int QT, int NW>
+__global__ __launch_bounds__(64 * NW) void attn_prefill_lds_kernel(AttnArgs a, int n_items) {
+  constexpr int ROWS_WG = 16 * QT * NW;                  // NW waves, each with QT 16-row tiles
+  constexpr int BPI = ITEM_ROWS / ROWS_WG;               // workgroups per item
+  static_assert(ITEM_ROWS % ROWS_WG == 0, "a workgroup's rows must divide an item");
   constexpr int NDT = DPAD / 16, NQS = DPAD / VK_SLAB;
   constexpr int EB = (int)sizeof(elem_t);
   constexpr int KRB = DPAD * EB, CK = KRB / 16;          // key row: bytes, 16-byte columns
   constexpr int VRB = TILE_KEYS * EB, CV = VRB / 16;     // value row (one d index, 64 keys)
   constexpr int KT_BYTES = TILE_KEYS * KRB, STAGE = 2 * KT_BYTES;   // value tile: DPAD * VRB, the same
-  constexpr int NI = CK / 4;                             // wave-level loads per wave for keys; as many for values
+  constexpr int NI = CK / NW;                            // wave-level loads per wave for keys; as many for values
   constexpr int KMASK = CK >= 16 ? 15 : CK - 1;
-  static_assert(CK % 4 == 0 && CK >= 8, "head size too small for this kernel");
+  static_assert(CK % NW == 0, "head size too small for this kernel");
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];   // [2][key tile, value tile]
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // The wave's index as a scalar: what depends on it alone then branches for the wave as a whole.
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r16 = lane & 15, g = lane >> 4;
-  // Workgroups that run together on a chip quarter (every 8th index) get the q heads of the same
-  // item, which share keys; long items first.
-  const int total = n_items * a.nq;
+  // Workgroup i runs on chip part i % 8, each with a cache of its own.  Long items first (items
+  // are in ascending row order and later rows see more keys), dealt to the parts in turn, and the q
+  // heads of an item, which share keys, one after the other on the same part.
   const int lin = blockIdx.x;
-  const int v = total % 8 == 0 ? (lin & 7) * (total >> 3) + (lin >> 3) : lin;
-  const int item = n_items - 1 - v / a.nq, head = v % a.nq;
+  const int n_blocks = n_items * BPI;
+  int rank, head;            // rank: 0 for the last rows of the last item
+  if (n_blocks % 8 == 0) {
+    const int j = lin >> 3;
+    rank = (j / a.nq) * 8 + (lin & 7);
+    head = j % a.nq;
+  } else {
+    rank = lin / a.nq;
+    head = lin % a.nq;
+  }
+  const int block = n_blocks - 1 - rank;
+  const int item = block / BPI;
   const int kvh = head / (a.nq / a.nkv);
-  const int seq = a.items[2 * item], q_off0 = a.items[2 * item + 1];
+  const int seq = a.items[2 * item], q_off0 = a.items[2 * item + 1] + (block % BPI) * ROWS_WG;
   const int q_begin = a.cu_q[seq], q_len = a.cu_q[seq + 1] - q_begin;
+  if (q_off0 >= q_len) return;                           // the item ends before this workgroup's rows
   const int k_len = a.k_len[seq];
-  const int rows_item = min(ITEM_ROWS, q_len - q_off0);
+  const int rows_item = min(ROWS_WG, q_len - q_off0);    // this workgroup's rows
   const int pos_item = k_len - q_len + q_off0;           // position of the item's first row
   const int item_lo = a.window > 0 ? max(0, pos_item - a.window + 1) : 0;
   const int tile_lo = item_lo / TILE_KEYS, tile_hi = (pos_item + rows_item - 1) / TILE_KEYS;
 
   // ---- this wave's rows ----
-  const int rows_wave = min(32, rows_item - 32 * wave);  // <= 0: the wave only helps to load
-  const int pos_wave = pos_item + 32 * wave;
+  const int rows_wave = min(16 * QT, rows_item - 16 * QT * wave);  // <= 0: the wave only helps to load
+  const int pos_wave = pos_item + 16 * QT * wave;
   const int wave_lo = a.window > 0 ? max(0, pos_wave - a.window + 1) : 0;
   const int wtile_lo = wave_lo / TILE_KEYS, wtile_hi = rows_wave > 0 ? (pos_wave + rows_wave - 1) / TILE_KEYS : -1;
-  bool row_ok[2];
-  int pos[2], lo[2], tok[2];
-  frag_t qf[2][NQS];
+  bool row_ok[QT];
+  int pos[QT], lo[QT], tok[QT];
+  frag_t qf[QT][NQS];
 #pragma unroll
-  for (int qt = 0; qt < 2; ++qt) {
+  for (int qt = 0; qt < QT; ++qt) {
     row_ok[qt] = 16 * qt + r16 < rows_wave;
     pos[qt] = pos_wave + 16 * qt + r16;
     lo[qt] = a.window > 0 ? max(0, pos[qt] - a.window + 1) : 0;
-    tok[qt] = q_begin + q_off0 + 32 * wave + 16 * qt + r16;
+    tok[qt] = q_begin + q_off0 + 16 * QT * wave + 16 * qt + r16;
     load_q<NQS>(a, tok[qt], head, row_ok[qt], g, qf[qt]);
   }
 
@@ -409,7 +444,7 @@ __global__ __launch_bounds__(256) void attn_prefill_lds_kernel(AttnArgs a, int n
   int koff[NI], voff[NI];       // element offsets from the tile's first key (keys) or from its page row 0 (values)
 #pragma unroll
   for (int j = 0; j < NI; ++j) {
-    const int instr = wave + 4 * j;                        // 1 KB of the tile each
+    const int instr = wave + NW * j;                       // 1 KB of the tile each
     const int krow = instr * (1024 / KRB) + lane / CK;     // key within the tile
     const int kcol = (lane % CK) ^ (key_swz(krow) & KMASK);
     koff[j] = krow * DPAD + kcol * VK_VEC;
@@ -426,15 +461,15 @@ __global__ __launch_bounds__(256) void attn_prefill_lds_kernel(AttnArgs a, int n
     unsigned char* dst = lds + stage * STAGE + wave * 1024;
 #pragma unroll
     for (int j = 0; j < NI; ++j) {
-      load_to_lds16(kt + koff[j], dst + j * 4096);
-      load_to_lds16(vt + voff[j], dst + KT_BYTES + j * 4096);
+      load_to_lds16(kt + koff[j], dst + j * NW * 1024);
+      load_to_lds16(vt + voff[j], dst + KT_BYTES + j * NW * 1024);
     }
   };
 
-  float M[2], L[2], Ms[2], Ls[2];
-  f32x4 ACC[2][NDT], As[2][NDT];
+  float M[QT], L[QT], Ms[QT], Ls[QT];
+  f32x4 ACC[QT][NDT], As[QT][NDT];
 #pragma unroll
-  for (int qt = 0; qt < 2; ++qt) {
+  for (int qt = 0; qt < QT; ++qt) {
     M[qt] = Ms[qt] = -INFINITY;
     L[qt] = Ls[qt] = 0.f;
 #pragma unroll
@@ -452,7 +487,7 @@ __global__ __launch_bounds__(256) void attn_prefill_lds_kernel(AttnArgs a, int n
       const unsigned char* kl = lds + stage * STAGE;
       const unsigned char* vl = kl + KT_BYTES;
       // ---- scores of both row tiles ----
-      float sc[2][S_PER_LANE];
+      float sc[QT][S_PER_LANE];
 #pragma unroll
       for (int sub = 0; sub < S_PER_LANE / 4; ++sub) {
         const int krow = key_row_of(sub, r16);
@@ -462,7 +497,7 @@ __global__ __launch_bounds__(256) void attn_prefill_lds_kernel(AttnArgs a, int n
 #pragma unroll
         for (int s = 0; s < NQS; ++s) kf[s] = *reinterpret_cast<const frag_t*>(kr + (((s * 4 + g) ^ sw) << 4));
 #pragma unroll
-        for (int qt = 0; qt < 2; ++qt) {
+        for (int qt = 0; qt < QT; ++qt) {
           f32x4 s4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int s = 0; s < NQS; ++s) s4 = mma_slab(kf[s], qf[qt][s], s4);
@@ -473,48 +508,60 @@ __global__ __launch_bounds__(256) void attn_prefill_lds_kernel(AttnArgs a, int n
         }
       }
       // ---- each row's own statistics of this tile, and how they fold into the segment's ----
-      frag_t pf[2][KEY_SLABS];
-      float ca[2], cb[2];
-      bool some[2];
+      frag_t pf[QT][KEY_SLABS];
+      float ca[QT], cb[QT];
+      bool some[QT], all_some[QT];
 #pragma unroll
-      for (int qt = 0; qt < 2; ++qt) {
+      for (int qt = 0; qt < QT; ++qt) {
+        const bool full = rows_wave >= 16 * qt + 16 && kb + TILE_KEYS - 1 <= pos_wave + 16 * qt &&
+                          kb >= (a.window > 0 ? max(0, pos_wave + 16 * qt + 15 - a.window + 1) : 0);
         float m_t, l_t, Mn;
-        tile_softmax(sc[qt], kb, g, row_ok[qt], lo[qt], pos[qt], a.scale_log2, m_t, l_t, pf[qt]);
+        tile_softmax(sc[qt], kb, g, row_ok[qt], lo[qt], pos[qt], a.scale_log2, full, m_t, l_t, pf[qt]);
         some[qt] = m_t > -INFINITY;
+        all_some[qt] = __all(some[qt]);
         fold_scales(Ms[qt], m_t, Mn, ca[qt], cb[qt]);
         if (some[qt]) {
           Ls[qt] = fold1(Ls[qt], l_t, ca[qt], cb[qt]);
           Ms[qt] = Mn;
         }
       }
-      // ---- P V from zero, folded into the segment's sum column block by column block ----
+      // ---- P V from zero, folded into the segment's sum column block by column block: fold()'s
+      // arithmetic.  When every row of the wave has a key in the tile, which is the rule, the loop
+      // has no branch and no select inside, so that the reads from LDS, the MFMAs and the folds of
+      // different column blocks overlap.
       const bool edge = kb + TILE_KEYS > k_len || kb < wave_lo;
+      auto pv = [&](auto plain_tag, int qt) {
+        constexpr bool PLAIN = decltype(plain_tag)::value;
 #pragma unroll
-      for (int dt = 0; dt < NDT; ++dt) {
-        const int vrow = dt * 16 + r16;
-        const unsigned char* vr = vl + vrow * VRB;
-        const int sw = val_swz(vrow);
-        frag_t vf[KEY_SLABS];
+        for (int dt = 0; dt < NDT; ++dt) {
+          const int vrow = dt * 16 + r16;
+          const unsigned char* vr = vl + vrow * VRB;
+          const int sw = val_swz(vrow);
+          frag_t vf[KEY_SLABS];
 #pragma unroll
-        for (int ks = 0; ks < KEY_SLABS; ++ks) vf[ks] = *reinterpret_cast<const frag_t*>(vr + (((ks * 4 + g) ^ sw) << 4));
-        if (edge) zero_unowned(vf, kb, g, wave_lo, k_len);
-#pragma unroll
-        for (int qt = 0; qt < 2; ++qt) {
+          for (int ks = 0; ks < KEY_SLABS; ++ks) vf[ks] = *reinterpret_cast<const frag_t*>(vr + (((ks * 4 + g) ^ sw) << 4));
+          if (!PLAIN && edge) zero_unowned(vf, kb, g, wave_lo, k_len);
           f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int ks = 0; ks < KEY_SLABS; ++ks) acc = mma_slab(vf[ks], pf[qt][ks], acc);
-          if (some[qt]) {
-            As[qt][dt].x = fold1(As[qt][dt].x, acc.x, ca[qt], cb[qt]);
-            As[qt][dt].y = fold1(As[qt][dt].y, acc.y, ca[qt], cb[qt]);
-            As[qt][dt].z = fold1(As[qt][dt].z, acc.z, ca[qt], cb[qt]);
-            As[qt][dt].w = fold1(As[qt][dt].w, acc.w, ca[qt], cb[qt]);
+          f32x4& A = As[qt][dt];
+          if (PLAIN || some[qt]) {
+            A.x = fold1(A.x, acc.x, ca[qt], cb[qt]);
+            A.y = fold1(A.y, acc.y, ca[qt], cb[qt]);
+            A.z = fold1(A.z, acc.z, ca[qt], cb[qt]);
+            A.w = fold1(A.w, acc.w, ca[qt], cb[qt]);
           }
         }
+      };
+#pragma unroll
+      for (int qt = 0; qt < QT; ++qt) {
+        if (!edge && all_some[qt]) pv(std::true_type{}, qt);
+        else pv(std::false_type{}, qt);
       }
     }
     if ((t + 1) % SEG_TILES == 0 || t == tile_hi) {        // the segment is complete
 #pragma unroll
-      for (int qt = 0; qt < 2; ++qt) {
+      for (int qt = 0; qt < QT; ++qt) {
         fold<NDT>(M[qt], L[qt], ACC[qt], Ms[qt], Ls[qt], As[qt]);
         Ms[qt] = -INFINITY;
         Ls[qt] = 0.f;
@@ -524,7 +571,7 @@ __global__ __launch_bounds__(256) void attn_prefill_lds_kernel(AttnArgs a, int n
     }
   }
 #pragma unroll
-  for (int qt = 0; qt < 2; ++qt) {
+  for (int qt = 0; qt < QT; ++qt) {
     if (row_ok[qt]) {
       const float inv = L[qt] > 0.f ? 1.0f / L[qt] : 0.f;
       elem_t* orow = a.out + ((int64_t)tok[qt] * a.nq + head) * a.d;
@@ -684,6 +731,11 @@ int vk_attn_segment_keys(void) { return TILE_KEYS * SEG_TILES; }
 
 int vk_attn_item_rows(void) { return ITEM_ROWS; }
 
+// For measurements: 0 is the default shape of the workgroups of the prompt kernel, 14 and 24 are the
+// others (row tiles per wave * 10 + waves).  The result is the same bits.
+static int vk_prefill_variant = 0;
+void vk_attn_set_prefill_variant(int v) { vk_prefill_variant = v; }
+
 // 1 if prompt rows of this shape go through the kernel that shares key tiles in LDS.
 int vk_attn_prefill_shares_tiles(int d, int P) {
   return (d == 64 || d == 128 || d == 256) && P >= TILE_KEYS && 4 * TILE_KEYS * d * (int)sizeof(elem_t) <= 128 * 1024;
@@ -704,6 +756,7 @@ int vk_paged_attention(elem_t* out, const elem_t* q, const elem_t* kc, const ele
   VK_REQUIRE(d >= 16 && d <= 256 && d % 16 == 0, "attention: head size %d must be a multiple of 16 in 16..256", d);
   VK_REQUIRE(P >= 8 && (P & (P - 1)) == 0, "attention: page size %d must be a power of two >= 8", P);
   VK_REQUIRE(window >= 0, "attention: window %d must not be negative", window);
+  VK_REQUIRE(scale > 0.f, "attention: the score scale must be positive");
   VK_REQUIRE(mode >= 0 && mode <= 2, "attention: unknown mode %d", mode);
   if (n_items <= 0) return 0;
   AttnArgs a;
@@ -713,21 +766,24 @@ int vk_paged_attention(elem_t* out, const elem_t* q, const elem_t* kc, const ele
   a.part_ml = nullptr; a.part_acc = nullptr;
   const int G = nq / nkv;
   if (mode == 0 && vk_attn_prefill_shares_tiles(d, P)) {
-    VK_REQUIRE((int64_t)n_items * nq < (1ll << 31), "attention: too many prompt items");
+    VK_REQUIRE((int64_t)n_items * (ITEM_ROWS / 16) * nq < (1ll << 31), "attention: too many prompt items");
     const size_t smem = (size_t)4 * TILE_KEYS * d * sizeof(elem_t);
-#define PREFILL_LDS(DP)                                                                              \
+#define PREFILL_LDS(DP, QT, NW)                                                                      \
   do {                                                                                               \
     static bool raised = false;                                                                      \
     if (!raised) {                                                                                   \
-      (void)hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<DP>,                            \
+      (void)hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<DP, QT, NW>,                    \
                                 hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);             \
       raised = true;                                                                                 \
     }                                                                                                \
-    attn_prefill_lds_kernel<DP><<<n_items * nq, 256, smem, st>>>(a, n_items);                        \
+    attn_prefill_lds_kernel<DP, QT, NW><<<n_items * (ITEM_ROWS / (16 * QT * NW)) * nq, 64 * NW, smem, st>>>(a, n_items); \
   } while (0)
-    if (d == 64) PREFILL_LDS(64);
-    else if (d == 128) PREFILL_LDS(128);
-    else PREFILL_LDS(256);
+    // Eight waves of one row tile each measured best on long contexts (MI355X, head size 128); four
+    // waves are a few per cent better on short ones, two row tiles per wave need too many registers.
+    const int v = vk_prefill_variant;
+    if (d == 64) { if (v == 14) PREFILL_LDS(64, 1, 4); else if (v == 24) PREFILL_LDS(64, 2, 4); else PREFILL_LDS(64, 1, 8); }
+    else if (d == 128) { if (v == 14) PREFILL_LDS(128, 1, 4); else if (v == 24) PREFILL_LDS(128, 2, 4); else PREFILL_LDS(128, 1, 8); }
+    else { if (v == 14) PREFILL_LDS(256, 1, 4); else if (v == 24) PREFILL_LDS(256, 2, 4); else PREFILL_LDS(256, 1, 8); }
 #undef PREFILL_LDS
     return vk_check_launch("attention (prompt rows, shared tiles)");
   }

@@ -54,6 +54,21 @@ __device__ __forceinline__ float wave_sum_xor(float v) {
   return v;
 }
 
+// The values of lanes l ^ 16 and l ^ 32 (what __shfl_xor gives), through the row and half swaps of
+// gfx950, which stay in the vector unit instead of going through LDS.
+__device__ __forceinline__ float lane_xor16(float v) {
+  const unsigned u = __builtin_bit_cast(unsigned, v);
+  // Rows of 16 lanes r0 r1 r2 r3: the swap leaves (r0 r0 r2 r2, r1 r1 r3 r3).
+  const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  return __builtin_bit_cast(float, (threadIdx.x & 16) ? r[0] : r[1]);
+}
+__device__ __forceinline__ float lane_xor32(float v) {
+  const unsigned u = __builtin_bit_cast(unsigned, v);
+  // Halves h0 h1: the swap leaves (h0 h0, h1 h1).
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __builtin_bit_cast(float, (threadIdx.x & 32) ? r[0] : r[1]);
+}
+
 __device__ __forceinline__ float wave_max_xor(float v) {
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, VK_WAVE));
