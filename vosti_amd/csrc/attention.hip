@@ -141,7 +141,7 @@ __device__ __forceinline__ void zero_unowned(frag_t (&vf)[KEY_SLABS], int kb, in
 }
 
 // One tile, reduced on its own: m, l and acc[NDT] of this lane's row.
-template <int NDT, int NQS>
+template <int NDT, int NQS, bool V_LATE>
 __device__ __forceinline__ void tile_partial(const RowCtx& c, const frag_t (&qf)[NQS], int kb, float& m_t, float& l_t,
                                              f32x4 (&acc)[NDT]) {
   const int d = c.d, P = c.P, r16 = c.r16, g = c.g;
@@ -179,6 +179,25 @@ __device__ __forceinline__ void tile_partial(const RowCtx& c, const frag_t (&qf)
       }
     }
   }
+  // ---- value fragments ----
+  frag_t vf[NDT][KEY_SLABS];
+  auto load_values = [&]() {
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) {
+      if (dt * 16 < d) {
+#pragma unroll
+        for (int ks = 0; ks < KEY_SLABS; ++ks) {
+          const int k0 = kb + ks * VK_SLAB + g * VK_VEC;
+          const int kk = k0 <= last_key ? k0 : kb;     // a whole vector inside a page of this sequence
+          const elem_t* vrow = (one_page ? vpage : c.vbase + c.bt[kk >> lp] * c.page_stride) +
+                               (int64_t)(dt * 16 + r16) * P + (kk & (P - 1));
+          vf[dt][ks] = *reinterpret_cast<const frag_t*>(vrow);
+        }
+      }
+    }
+  };
+  // A wave that has the SIMD nearly to itself (few decoded tokens) asks for everything at once.
+  if (!V_LATE) load_values();
   // ---- scores S^T[key, row] = K Q^T ----
   float sc[S_PER_LANE];
 #pragma unroll
@@ -192,22 +211,11 @@ __device__ __forceinline__ void tile_partial(const RowCtx& c, const frag_t (&qf)
     sc[4 * sub + 2] = s4.z;
     sc[4 * sub + 3] = s4.w;
   }
-  // ---- value fragments: requested once the key fragments' registers are free again, so that more
-  // waves fit a SIMD; their latency passes behind the softmax arithmetic and the other waves ----
-  __builtin_amdgcn_sched_barrier(0);
-  frag_t vf[NDT][KEY_SLABS];
-#pragma unroll
-  for (int dt = 0; dt < NDT; ++dt) {
-    if (dt * 16 < d) {
-#pragma unroll
-      for (int ks = 0; ks < KEY_SLABS; ++ks) {
-        const int k0 = kb + ks * VK_SLAB + g * VK_VEC;
-        const int kk = k0 <= last_key ? k0 : kb;     // a whole vector inside a page of this sequence
-        const elem_t* vrow = (one_page ? vpage : c.vbase + c.bt[kk >> lp] * c.page_stride) +
-                             (int64_t)(dt * 16 + r16) * P + (kk & (P - 1));
-        vf[dt][ks] = *reinterpret_cast<const frag_t*>(vrow);
-      }
-    }
+  if (V_LATE) {
+    // Requested once the key fragments' registers are free again, so that more waves fit a SIMD;
+    // the latency passes behind the softmax arithmetic and the other waves.
+    __builtin_amdgcn_sched_barrier(0);
+    load_values();
   }
   // ---- mask, maximum, probabilities; acc = V^T P^T from zero ----
   frag_t pf[KEY_SLABS];
@@ -324,7 +332,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a, int heads
     for (int t = max(tile_lo, seg * SEG_TILES); t <= t_end; ++t) {
       float m_t, l_t;
       f32x4 acc[NDT];
-      tile_partial<NDT, NQS>(c, qf, t * TILE_KEYS, m_t, l_t, acc);
+      tile_partial<NDT, NQS, true>(c, qf, t * TILE_KEYS, m_t, l_t, acc);
       fold<NDT>(Ms, Ls, As, m_t, l_t, acc);
     }
     fold<NDT>(M, L, ACC, Ms, Ls, As);
@@ -588,7 +596,7 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_lds_kernel(AttnArgs a, i
 
 // Decoded tokens: an item is one token; the 16 rows of a wave are up to 16 q
 // heads of one kv head.  Workgroup = one segment, wave = one tile of it.
-template <int DPAD>
+template <int DPAD, bool V_LATE>
 __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
   constexpr int NDT = DPAD / 16, NQS = DPAD / VK_SLAB;
   extern __shared__ __attribute__((aligned(16))) float smem[];
@@ -623,7 +631,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
     frag_t qf[NQS];
     load_q<NQS>(a, tok, head, c.row_ok, c.g, qf);
     f32x4 acc[NDT];
-    tile_partial<NDT, NQS>(c, qf, t * TILE_KEYS, m_t, l_t, acc);
+    tile_partial<NDT, NQS, V_LATE>(c, qf, t * TILE_KEYS, m_t, l_t, acc);
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt)
       if (dt * 16 < a.d) *reinterpret_cast<f32x4*>(&s_acc[wave][c.r16][dt * 16 + 4 * c.g]) = acc[dt];
@@ -802,17 +810,21 @@ int vk_paged_attention(elem_t* out, const elem_t* q, const elem_t* kc, const ele
   a.part_acc = scratch + (((int64_t)total_tokens * nq * nseg * 2 + 3) & ~(int64_t)3);
   const dim3 grid(n_items, nkv * ((G + 15) / 16), nseg);
   VK_REQUIRE(grid.y <= 65535 && nq <= 65535, "attention: too many heads");
-#define DECODE(DP)                                                                                   \
+#define DECODE(DP, LATE)                                                                             \
   do {                                                                                               \
     const size_t smem = (size_t)SEG_TILES * 16 * (DP + 2) * sizeof(float);                           \
     if (smem > 48 * 1024)                                                                            \
-      (void)hipFuncSetAttribute((const void*)attn_decode_kernel<DP>,                                 \
+      (void)hipFuncSetAttribute((const void*)attn_decode_kernel<DP, LATE>,                           \
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);              \
-    attn_decode_kernel<DP><<<grid, 256, smem, st>>>(a);                                              \
+    attn_decode_kernel<DP, LATE><<<grid, 256, smem, st>>>(a);                                        \
   } while (0)
-  if (d <= 64) DECODE(64);
-  else if (d <= 128) DECODE(128);
-  else DECODE(256);
+  // With few workgroups a wave asks for keys and values together; with many, the values wait until
+  // the keys' registers are free, so that more waves fit a SIMD (measured on MI355X: the two cross
+  // between 8 and 64 tokens of 2,000 keys).
+  const bool late = (int64_t)grid.x * grid.y * grid.z > 1024;
+  if (d <= 64) { if (late) DECODE(64, true); else DECODE(64, false); }
+  else if (d <= 128) { if (late) DECODE(128, true); else DECODE(128, false); }
+  else { if (late) DECODE(256, true); else DECODE(256, false); }
 #undef DECODE
   if (vk_check_launch("attention (decoded rows)")) return 1;
   attn_combine_kernel<<<dim3(n_items, nq), 64, 0, st>>>(a);
