@@ -114,6 +114,26 @@ def test_long_decoding_equals_whole_prompt(tiny_dirs, dtype_name):
     assert e.kernels.sample(logits).cpu().tolist() == out
 
 
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_schedule_stress(tiny_dirs, dtype_name):
+    """Prompts of 17 to 385 tokens around page and tile edges, 16 new tokens each, four rows and 128
+    tokens a step, staggered arrival (the reference's schedule stress,
+    scripts/determinism_tests/schedule_stress.py:20-106): with many pages or few, with or without graph
+    replay, every request gets the tokens of a run on its own."""
+    from vosti_amd.sampling import SamplingParams
+    ps = prompts("C", [17, 63, 64, 65, 127, 129, 257, 385], seed=12)
+    sp = SamplingParams(max_tokens=16)
+    arrivals = [0, 0, 2, 4, 8, 12, 16, 20]
+    alone = [engine(tiny_dirs["C"], dtype_name, num_pages=8, page_size=64, max_num_seqs=1, graphs=False).generate([p], sp)[0]
+             for p in ps]
+    for pages, graphs in ((128, True), (32, False), (14, True)):
+        e = engine(tiny_dirs["C"], dtype_name, num_pages=pages, page_size=64, max_num_seqs=4, max_num_batched_tokens=128,
+                   graphs=graphs)
+        outs = e.generate(ps, sp, arrival_steps=arrivals)
+        assert outs == alone, (pages, graphs)
+        assert e.cache.num_requests() == 0 and e.cache.check() == ""
+
+
 def test_pages_run_out_through_the_engine(tiny_dirs):
     """So few pages that requests are preempted and recomputed: the tokens are still those of a roomy run."""
     from vosti_amd.cache import OutOfPages

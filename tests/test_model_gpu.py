@@ -20,7 +20,7 @@ DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
 # bfloat16: the plain implementation rounds where the engine does, but a sum taken in another
 # order can land on the neighbouring bfloat16 (2^-8 relative), and layers carry that on.
 TOL = {"float32": dict(rtol=1e-4, atol=2e-5), "bfloat16": dict(rtol=3e-2, atol=3e-2)}
-LENGTHS = {"A": [1, 7, 33, 64, 100, 128], "B": [2, 17, 63, 65, 120, 129, 200, 256]}
+LENGTHS = {"A": [1, 7, 33, 64, 100, 128], "B": [2, 17, 63, 65, 120, 129, 200, 256], "C": [3, 64, 65, 130, 257, 300, 512]}
 
 
 def prompts_for(name):
@@ -130,7 +130,7 @@ def cut_mixed(prompts, page, max_live=4, seed=5):
 
 
 @pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_every_cutting(tiny_dirs, plain_logits, name, dtype_name):
     prompts = prompts_for(name)
     page = TINY[name][1]

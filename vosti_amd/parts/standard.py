@@ -189,7 +189,7 @@ class Attention(Mixer):
             nseg = -(-ctx.max_decode_k_len // SEGMENT_KEYS)
             scratch = ctx.attn_scratch(k.attn_scratch_floats(T, nq, d, nseg))
             k.paged_attention(q, cache.k, cache.v, tables.block_table, ctx.cu_q, ctx.k_len, ctx.decode_items, mode=1,
-                              scale=self.scale, window=self.window, max_k_len=ctx.max_k_len, nseg=nseg,
+                              scale=self.scale, window=self.window, max_k_len=ctx.max_decode_k_len, nseg=nseg,
                               scratch=scratch, out=out)
         return k.gemm(out.view(T, nq * d), self.w_o)
 
