@@ -30,7 +30,8 @@ def rand(shape, dtype, seed, scale=1.0):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,N,K", [(1, 64, 64), (5, 503, 96), (17, 224, 96), (64, 256, 224), (16, 48, 520),
                                    (65, 130, 520), (130, 96, 1032), (300, 520, 2056), (8, 40, 4104),
-                                   (8, 4100, 1024), (3, 72, 512), (33, 200, 1536), (64, 4096, 4608), (17, 90, 5120)])
+                                   (8, 4100, 1024), (3, 72, 512), (33, 200, 1536), (64, 4096, 4608), (17, 90, 5120),
+                                   (40, 6200, 1024), (64, 6144, 512), (23, 24, 2048)])
 def test_gemm(dtype, M, N, K):
     k = kern(dtype)
     a, w = rand((M, K), dtype, 1), rand((N, K), dtype, 2, 0.1)
@@ -38,8 +39,9 @@ def test_gemm(dtype, M, N, K):
     got_t = k.gemm(a.cuda(), w.cuda(), kernel=2)
     torch.testing.assert_close(got_t.float().cpu(), ref.to(dtype).float(), **tol(dtype))
     if M <= 64:
-        got_s = k.gemm(a.cuda(), w.cuda(), kernel=1)
-        assert torch.equal(got_s, got_t), "the skinny and the tiled kernel must agree bitwise"
+        for code in (1, 7, 0):    # one and two weight tiles per workgroup, and the kernel chosen by size
+            got_s = k.gemm(a.cuda(), w.cuda(), kernel=code)
+            assert torch.equal(got_s, got_t), f"the skinny kernel {code} and the tiled kernel must agree bitwise"
     # A row of a batch equals the same row alone, bitwise.
     for r in {0, M // 2, M - 1}:
         one = k.gemm(a[r:r + 1].cuda(), w.cuda())

@@ -135,25 +135,29 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_kernel(elem_t* __re
 // a loaded value makes the compiler wait for it at once; and with RES (K <= 4096,
 // one 16-row activation tile) a wave keeps the activations of its chunk in
 // registers for the whole kernel.  One barrier per round of eight chunks.
-template <int MT, int W, bool RES>
+template <int MT, int W, bool RES, int NT>
 __global__ __launch_bounds__(64 * SK_WAVES) void gemm_stream_kernel(elem_t* __restrict__ out,
                                                                     const elem_t* __restrict__ act,
                                                                     const elem_t* __restrict__ w, int M, int N, int K,
                                                                     int64_t lda, int64_t ldo, int out_vec_ok) {
+  // NT: 16-row weight tiles per workgroup.  With several activation tiles every workgroup reads all
+  // activations once, M * K elements beside its 16 * NT * K weights: more weight rows per workgroup
+  // keep that traffic, which comes from the second-level cache, in proportion.
   static_assert(KC_SLABS % W == 0, "the window must divide a chunk");
   static_assert(!RES || MT == 1, "resident activations are for one activation tile");
-  __shared__ f32x4 part[2][SK_WAVES][MT][64];
+  static_assert(NT * MT <= SK_WAVES, "one wave adds up each output tile");
+  __shared__ f32x4 part[2][SK_WAVES][NT * MT][64];
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r16 = lane & 15, kg = lane >> 4;
   const int nchunks = K / KC;
-  const int ntiles = (N + 15) / 16;
+  const int ntiles = (N + 16 * NT - 1) / (16 * NT);     // tile: NT * 16 weight rows
 
   const elem_t* arow[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) arow[mt] = act + (int64_t)min(mt * 16 + r16, M - 1) * lda + kg * VK_VEC;
 
-  frag_t wbuf[W], abuf[RES ? KC_SLABS : W][MT];
+  frag_t wbuf[W][NT], abuf[RES ? KC_SLABS : W][MT];
   if (RES) {
     if (wave < nchunks) {
 #pragma unroll
@@ -162,7 +166,9 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_stream_kernel(elem_t* __re
   }
   auto issue = [&](int tile, int c, int s, int slot) {
     const int k = c * KC + s * VK_SLAB;
-    wbuf[slot] = *reinterpret_cast<const frag_t*>(w + (int64_t)min(tile * 16 + r16, N - 1) * K + kg * VK_VEC + k);
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+      wbuf[slot][nt] = *reinterpret_cast<const frag_t*>(w + (int64_t)min((tile * NT + nt) * 16 + r16, N - 1) * K + kg * VK_VEC + k);
     if (!RES) {
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) abuf[slot][mt] = *reinterpret_cast<const frag_t*>(arow[mt] + k);
@@ -179,34 +185,41 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_stream_kernel(elem_t* __re
     f32x4 total = {0.f, 0.f, 0.f, 0.f};
     for (int base = 0; base < nchunks; base += SK_WAVES) {
       const int c = base + wave;
-      f32x4 acc[MT];
+      f32x4 acc[NT][MT];
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
       if (c < nchunks) {
         // What this wave streams next: its next chunk of this tile, else its first chunk of the next tile.
-        int nt = tile, nc = c + SK_WAVES;
+        int nt_ = tile, nc = c + SK_WAVES;
         if (nc >= nchunks) {
-          nt = tile + gridDim.x;
+          nt_ = tile + gridDim.x;
           nc = wave;
         }
-        const bool has_next = nt < ntiles;
+        const bool has_next = nt_ < ntiles;
 #pragma unroll
         for (int i = 0; i < KC_SLABS; ++i) {
           const int slot = i % W;
-          const frag_t fw = wbuf[slot];
-          frag_t fa[MT];
+          frag_t fw[NT], fa[MT];
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) fw[nt] = wbuf[slot][nt];
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt) fa[mt] = RES ? abuf[i][mt] : abuf[slot][mt];
           if (i + W < KC_SLABS) issue(tile, c, i + W, slot);
-          else if (has_next) issue(nt, nc, i + W - KC_SLABS, slot);
+          else if (has_next) issue(nt_, nc, i + W - KC_SLABS, slot);
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt) acc[mt] = mma_slab(fw, fa[mt], acc[mt]);
+          for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = mma_slab(fw[nt], fa[mt], acc[nt][mt]);
         }
       }
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) part[parity][wave][mt][lane] = acc[mt];
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) part[parity][wave][nt * MT + mt][lane] = acc[nt][mt];
       __syncthreads();
-      if (wave < MT) {
+      if (wave < NT * MT) {
         for (int w2 = 0; w2 < SK_WAVES; ++w2) {
           if (base + w2 < nchunks) {
             const f32x4 p = part[parity][w2][wave][lane];
@@ -216,7 +229,8 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_stream_kernel(elem_t* __re
       }
       parity ^= 1;
     }
-    if (wave < MT) store_out4(out, ldo, wave * 16 + r16, tile * 16 + 4 * kg, M, N, total, out_vec_ok);
+    if (wave < NT * MT)
+      store_out4(out, ldo, (wave % MT) * 16 + r16, (tile * NT + wave / MT) * 16 + 4 * kg, M, N, total, out_vec_ok);
   }
 }
 
@@ -557,8 +571,9 @@ static int launch_pipe(elem_t* out, const elem_t* act, const elem_t* w, int M, i
 // ==================================================================== host
 extern "C" {
 
-// kernel: 0 = choose by M, 1 = skinny (M <= 64), 2 = tiled (pipelined if K allows), 3 = tiled through
-// registers, 4..6 = pipelined with 2..4 stages (for measurements).  The result does not depend on the choice.
+// kernel: 0 = choose by size, 1 = skinny (M <= 64), 2 = tiled (pipelined if K allows), 3 = tiled through
+// registers, 4..6 = pipelined with 2..4 stages, 7 = skinny with two weight tiles per workgroup where it has
+// such a variant (for measurements and tests).  The result does not depend on the choice.
 int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K, int64_t lda, int64_t ldo,
             int kernel, hipStream_t st) {
   VK_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
@@ -567,35 +582,42 @@ int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K
              (long long)lda, VK_VEC);
   VK_REQUIRE(ldo >= N, "gemm: output row stride %lld is smaller than N=%d", (long long)ldo, N);
   VK_REQUIRE(((uintptr_t)act % 16) == 0 && ((uintptr_t)w % 16) == 0, "gemm: operands must be 16-byte aligned");
-  VK_REQUIRE(kernel >= 0 && kernel <= 6, "gemm: unknown kernel %d", kernel);
+  VK_REQUIRE(kernel >= 0 && kernel <= 7, "gemm: unknown kernel %d", kernel);
   if (M == 0) return 0;
   const int vec_ok = (ldo % 4 == 0) && ((uintptr_t)out % 16 == 0);
-  // Measured on Qwen3-8B shapes: with more than 16 rows and many weight rows the pipelined kernel wins,
-  // with few weight rows it has too few workgroups and the streaming kernel does.
-  if (kernel == 0) kernel = (M <= 16 || (M <= 64 && N < 16384)) ? 1 : 2;
-  if (kernel == 1) {
+  // Measured on Qwen3-8B shapes (MI355X).  Up to 16 rows: the streaming kernel.  17 to 64 rows: the
+  // streaming kernel with two weight tiles per workgroup where that still leaves some 200 workgroups
+  // (6144 weight rows), with one tile below that, and the pipelined tile kernel for many weight rows
+  // and more than 32 rows.  More rows: the pipelined tile kernel.
+  if (kernel == 0) {
+    if (M <= 16) kernel = 1;
+    else if (M <= 64) kernel = (N >= 16384 && M > 32) ? 2 : (N >= 6144 ? 7 : 1);
+    else kernel = 2;
+  }
+  if (kernel == 1 || kernel == 7) {
     VK_REQUIRE(M <= 64, "gemm: the skinny kernel takes at most 64 rows, got %d", M);
     const int mt = (M + 15) / 16;
     const unsigned grid = (unsigned)((N + 15) / 16);
     if (K % KC == 0) {
-#define ST(MT, W, RES)                                                                                    \
+#define ST(MT, W, RES, NT)                                                                                \
   do {                                                                                                    \
     static int resident = 0; /* workgroups of this kernel that the device holds at once */               \
     if (resident == 0) {                                                                                  \
       int dev = 0, cus = 0, per_cu = 0;                                                                   \
       (void)hipGetDevice(&dev);                                                                           \
       (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);                      \
-      (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gemm_stream_kernel<MT, W, RES>,         \
+      (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gemm_stream_kernel<MT, W, RES, NT>,     \
                                                          64 * SK_WAVES, 0);                               \
       resident = (cus > 0 ? cus : 256) * (per_cu > 0 ? per_cu : 1);                                       \
     }                                                                                                     \
-    gemm_stream_kernel<MT, W, RES><<<grid < (unsigned)resident ? grid : (unsigned)resident, 64 * SK_WAVES, \
-                                     0, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok);                    \
+    const unsigned groups = (unsigned)((N + 16 * NT - 1) / (16 * NT));                                    \
+    gemm_stream_kernel<MT, W, RES, NT><<<groups < (unsigned)resident ? groups : (unsigned)resident,       \
+                                         64 * SK_WAVES, 0, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok); \
   } while (0)
-      if (mt == 1) { if (K <= SK_WAVES * KC) ST(1, 8, true); else ST(1, 8, false); }
-      else if (mt == 2) ST(2, 8, false);
-      else if (mt == 3) ST(3, 4, false);
-      else ST(4, 4, false);
+      if (mt == 1) { if (K <= SK_WAVES * KC) ST(1, 8, true, 1); else ST(1, 8, false, 1); }
+      else if (mt == 2) { if (kernel == 7) ST(2, 4, false, 2); else ST(2, 8, false, 1); }
+      else if (mt == 3) { if (kernel == 7) ST(3, 4, false, 2); else ST(3, 4, false, 1); }
+      else { if (kernel == 7) ST(4, 4, false, 2); else ST(4, 4, false, 1); }
 #undef ST
       return vk_check_launch("gemm_stream");
     }
