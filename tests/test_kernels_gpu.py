@@ -68,7 +68,7 @@ def test_gemm_refuses_bad_width(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("T,H", [(1, 64), (7, 96), (33, 100), (5, 4104), (3, 17)])
+@pytest.mark.parametrize("T,H", [(1, 64), (7, 96), (33, 100), (5, 4104), (3, 17), (4, 2048), (2, 12288), (9, 4096)])
 def test_rmsnorm_and_add(dtype, T, H):
     k = kern(dtype)
     x, r, w = rand((T, H), dtype, 1), rand((T, H), dtype, 2), (1 + 0.1 * rand((H,), torch.float32, 3)).to(dtype)

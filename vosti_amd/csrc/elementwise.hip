@@ -92,6 +92,65 @@ __global__ __launch_bounds__(NORM_THREADS) void rmsnorm_kernel(
   }
 }
 
+// The same computation with the row in registers: NV vectors of VEC elements per thread, for rows of up
+// to NV * NORM_THREADS vectors.  The sums are taken in the order of rmsnorm_kernel, so the bits are the same.
+template <int VEC, bool ADD, int NV>
+__global__ __launch_bounds__(NORM_THREADS) void rmsnorm_reg_kernel(
+    elem_t* __restrict__ out, elem_t* res_io, const elem_t* __restrict__ x, const void* __restrict__ w,
+    int w_is_f32, int H, int heads, int64_t x_tok_stride, int64_t out_tok_stride, float eps) {
+  __shared__ float red[4];
+  const int r = blockIdx.x;
+  const int tok = r / heads, head = r - tok * heads;
+  const elem_t* xr = x + tok * x_tok_stride + (int64_t)head * H;
+  elem_t* outr = out + tok * out_tok_stride + (int64_t)head * H;
+  elem_t* resr = ADD ? res_io + (int64_t)r * H : nullptr;
+  const int nv = H / VEC;
+
+  float a[NV][VEC], wv[NV][VEC];
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int v = threadIdx.x + j * NORM_THREADS;
+    if (v < nv) {
+      load_elems(xr + v * VEC, a[j]);
+      if (w_is_f32) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) wv[j][i] = static_cast<const float*>(w)[v * VEC + i];
+      } else {
+        load_elems(static_cast<const elem_t*>(w) + v * VEC, wv[j]);
+      }
+    }
+  }
+  float part = 0.f;
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int v = threadIdx.x + j * NORM_THREADS;
+    if (v < nv) {
+      if (ADD) {
+        float b[VEC];
+        load_elems(resr + v * VEC, b);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) a[j][i] = a[j][i] + b[i];
+        store_elems(resr + v * VEC, a[j]);
+      }
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) part = part + a[j][i] * a[j][i];
+    }
+  }
+  const float total = block_sum_256(part, red);
+  const float var = total / (float)H;
+  const float rr = rsqrtf(var + eps);
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int v = threadIdx.x + j * NORM_THREADS;
+    if (v < nv) {
+      float y[VEC];
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) y[i] = (a[j][i] * rr) * wv[j][i];
+      store_elems(outr + v * VEC, y);
+    }
+  }
+}
+
 // ------------------------------------------------------------------- SwiGLU
 template <int VEC>
 __global__ __launch_bounds__(256) void swiglu_kernel(elem_t* __restrict__ out, const elem_t* __restrict__ gu,
@@ -197,11 +256,22 @@ static int norm_launch(bool add, elem_t* out, elem_t* res_io, const elem_t* x, c
     rmsnorm_kernel<VEC, ADD><<<rows, NORM_THREADS, smem, st>>>(out, res_io, x, w, w_is_f32, H, heads, \
                                                                xs, os, eps);                          \
   } while (0)
-  if (add) {
+#define LAUNCH_REG(ADD, NV)                                                                                    \
+  rmsnorm_reg_kernel<VK_VEC, ADD, NV><<<rows, NORM_THREADS, 0, st>>>(out, res_io, x, w, w_is_f32, H, heads, xs, os, eps)
+  const int nv = H / VK_VEC;
+  if (vec && nv <= 4 * NORM_THREADS) {
+    // The row fits the registers of a workgroup: no trip through LDS.
+    if (add) {
+      if (nv <= NORM_THREADS) LAUNCH_REG(true, 1); else if (nv <= 2 * NORM_THREADS) LAUNCH_REG(true, 2); else LAUNCH_REG(true, 4);
+    } else {
+      if (nv <= NORM_THREADS) LAUNCH_REG(false, 1); else if (nv <= 2 * NORM_THREADS) LAUNCH_REG(false, 2); else LAUNCH_REG(false, 4);
+    }
+  } else if (add) {
     if (vec) LAUNCH(VK_VEC, true); else LAUNCH(1, true);
   } else {
     if (vec) LAUNCH(VK_VEC, false); else LAUNCH(1, false);
   }
+#undef LAUNCH_REG
 #undef LAUNCH
   return vk_check_launch("rmsnorm");
 }
