@@ -463,8 +463,8 @@ __device__ __forceinline__ void wait_vmcnt(int n) {
   }
 }
 
-template <int S>
-__global__ __launch_bounds__(256) void gemm_pipe_kernel(elem_t* __restrict__ out, const elem_t* __restrict__ act,
+template <int S, bool WHOLE>
+__global__ __launch_bounds__(256, 2) void gemm_pipe_kernel(elem_t* __restrict__ out, const elem_t* __restrict__ act,
                                                         const elem_t* __restrict__ w, int M, int N, int K,
                                                         int64_t lda, int64_t ldo, int out_vec_ok) {
   constexpr int TILE_BYTES = 128 * T_ROWB, STAGE_BYTES = 2 * TILE_BYTES;
@@ -510,7 +510,7 @@ __global__ __launch_bounds__(256) void gemm_pipe_kernel(elem_t* __restrict__ out
   for (int p = 0; p < S - 1; ++p)
     if (p < ntiles) issue(p);
 
-  for (int kt = 0; kt < ntiles; ++kt) {
+  auto step = [&](int kt) {
     // Tile kt has landed once at most the loads of the tiles after it are outstanding (8 per tile and wave).
     const int later = min(S - 2, ntiles - 1 - kt);
     wait_vmcnt(8 * later);
@@ -531,17 +531,31 @@ __global__ __launch_bounds__(256) void gemm_pipe_kernel(elem_t* __restrict__ out
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[i][j] = mma_slab(wf[i], af[j], acc[i][j]);
     }
-    if ((kt + 1) % T_CHUNK_TILES == 0 || kt + 1 == ntiles) {
+  };
+  auto close_chunk = [&]() {
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          total[i][j].x = total[i][j].x + acc[i][j].x;
-          total[i][j].y = total[i][j].y + acc[i][j].y;
-          total[i][j].z = total[i][j].z + acc[i][j].z;
-          total[i][j].w = total[i][j].w + acc[i][j].w;
-          acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-        }
+      for (int j = 0; j < 4; ++j) {
+        total[i][j].x = total[i][j].x + acc[i][j].x;
+        total[i][j].y = total[i][j].y + acc[i][j].y;
+        total[i][j].z = total[i][j].z + acc[i][j].z;
+        total[i][j].w = total[i][j].w + acc[i][j].w;
+        acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+      }
+  };
+  if (WHOLE) {
+    // K is whole chunks: the tiles of a chunk are written out one after the other, so that the chunk
+    // sums are touched between chunks only and need not move between register files in every tile.
+    for (int kt0 = 0; kt0 < ntiles; kt0 += T_CHUNK_TILES) {
+#pragma unroll
+      for (int u = 0; u < T_CHUNK_TILES; ++u) step(kt0 + u);
+      close_chunk();
+    }
+  } else {
+    for (int kt = 0; kt < ntiles; ++kt) {
+      step(kt);
+      if ((kt + 1) % T_CHUNK_TILES == 0 || kt + 1 == ntiles) close_chunk();
     }
   }
 
@@ -559,12 +573,14 @@ static int launch_pipe(elem_t* out, const elem_t* act, const elem_t* w, int M, i
   const size_t smem = (size_t)S * 2 * 128 * T_ROWB;
   static bool configured = false;
   if (!configured) {
-    (void)hipFuncSetAttribute((const void*)gemm_pipe_kernel<S>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    (void)hipFuncSetAttribute((const void*)gemm_pipe_kernel<S, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    (void)hipFuncSetAttribute((const void*)gemm_pipe_kernel<S, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     configured = true;
   }
   dim3 grid((N + 127) / 128, (M + 127) / 128);
   VK_REQUIRE(grid.y <= 65535, "gemm: too many rows (%d)", M);
-  gemm_pipe_kernel<S><<<grid, 256, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok);
+  if (K % KC == 0) gemm_pipe_kernel<S, true><<<grid, 256, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok);
+  else gemm_pipe_kernel<S, false><<<grid, 256, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok);
   return vk_check_launch("gemm_pipe");
 }
 

@@ -11,7 +11,7 @@
 //   store      kernels/triton_kernels/store_kv_cache.py:89-120   slot -1 writes nothing
 // The reference runs them as five launches (src/exec/dense_swiglu_decoder.rs:207-272).
 //
-// One wave per (token, head); lane l owns elements l, l+64, l+128, l+192.
+// One wave per (token, head) at a time; lane l owns elements l, l+64, l+128, l+192.
 #include "common.h"
 #include "vec.h"
 
@@ -31,80 +31,102 @@ struct QkvPostArgs {
   float eps;
 };
 
-__global__ __launch_bounds__(64) void qkv_post_kernel(QkvPostArgs a) {
-  __shared__ float y[256];
-  const int tok = blockIdx.x, hh = blockIdx.y, lane = threadIdx.x;
-  const int d = a.d;
-  const int kind = hh < a.nq ? 0 : (hh < a.nq + a.nkv ? 1 : 2);   // q, k, v
-  const elem_t* x = a.qkv + tok * a.row_stride + (int64_t)hh * d;
-  const void* w = kind == 0 ? a.q_w : (kind == 1 ? a.k_w : nullptr);
+// A workgroup has four waves and one token; wave w takes the heads first + w, first + w + 4, ... of the
+// workgroup's `per_wave` * 4 heads, so that a long step does not start a workgroup per head.
+__global__ __launch_bounds__(256) void qkv_post_kernel(QkvPostArgs a, int per_wave) {
+  __shared__ float ybuf[4][256];
+  const int tok = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float* y = ybuf[wave];
+  const int d = a.d, heads = a.nq + 2 * a.nkv;
+  const int rh = a.rot_half;
+  // With a rotation half of 64 or 128 elements the partner of an element is held by the same lane.
+  const bool in_lane = rh % 64 == 0;
+  const int shift = rh / 64;
+  int64_t trow = 0;
+  if (a.cos_t != nullptr) trow = (int64_t)a.positions[tok] * rh;
+  const int slot = a.slots != nullptr ? a.slots[tok] : -1;
+  for (int j = 0; j < per_wave; ++j) {
+    const int hh = (blockIdx.y * per_wave + j) * 4 + wave;
+    const bool live = hh < heads;            // the same number of barriers for every wave
+    const int kind = hh < a.nq ? 0 : (hh < a.nq + a.nkv ? 1 : 2);   // q, k, v
+    const elem_t* x = a.qkv + tok * a.row_stride + (int64_t)(live ? hh : 0) * d;
+    const void* w = kind == 0 ? a.q_w : (kind == 1 ? a.k_w : nullptr);
 
-  float xv[4];
-  float part = 0.f;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int c = lane + 64 * i;
-    xv[i] = c < d ? to_f32(x[c]) : 0.f;
-    part = part + xv[i] * xv[i];
-  }
-  if (w != nullptr) {
-    const float total = wave_sum_xor(part);
-    const float rr = rsqrtf(total / (float)d + a.eps);
+    float xv[4];
+    float part = 0.f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int c = lane + 64 * i;
-      if (c < d) xv[i] = round_to_elem((xv[i] * rr) * load_weight(w, a.w_is_f32, c));
+      xv[i] = c < d ? to_f32(x[c]) : 0.f;
+      part = part + xv[i] * xv[i];
     }
-  }
-  const bool rotate = a.cos_t != nullptr && kind != 2;
-  if (rotate) {
+    if (w != nullptr) {
+      const float total = wave_sum_xor(part);
+      const float rr = rsqrtf(total / (float)d + a.eps);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int c = lane + 64 * i;
-      if (c < d) y[c] = xv[i];
-    }
-    __syncthreads();
-    const int rh = a.rot_half;
-    const int64_t trow = (int64_t)a.positions[tok] * rh;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int c = lane + 64 * i;
-      if (c < rh) {
-        const float cs = to_f32(a.cos_t[trow + c]), sn = to_f32(a.sin_t[trow + c]);
-        xv[i] = y[c] * cs - y[c + rh] * sn;
-      } else if (c < 2 * rh) {
-        const float cs = to_f32(a.cos_t[trow + c - rh]), sn = to_f32(a.sin_t[trow + c - rh]);
-        xv[i] = y[c] * cs + y[c - rh] * sn;
+      for (int i = 0; i < 4; ++i) {
+        const int c = lane + 64 * i;
+        if (c < d) xv[i] = round_to_elem((xv[i] * rr) * load_weight(w, a.w_is_f32, c));
       }
     }
-  }
-  if (kind == 0) {
-    elem_t* o = a.q_out + ((int64_t)tok * a.nq + hh) * d;
+    const bool rotate = a.cos_t != nullptr && kind != 2;
+    if (a.cos_t != nullptr && !in_lane) {
+      if (rotate) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int c = lane + 64 * i;
-      if (c < d) o[c] = from_f32<elem_t>(xv[i]);
+        for (int i = 0; i < 4; ++i) {
+          const int c = lane + 64 * i;
+          if (c < d) y[c] = xv[i];
+        }
+      }
+      __syncthreads();
     }
-    return;
-  }
-  const int slot = a.slots[tok];
-  if (slot < 0) return;
-  const int page = slot / a.P, off = slot - page * a.P;
-  if (kind == 1) {
-    const int kh = hh - a.nq;
-    elem_t* o = a.kc + (((int64_t)page * a.nkv + kh) * a.P + off) * d;
+    if (rotate) {
+      float old[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int c = lane + 64 * i;
-      if (c < d) o[c] = from_f32<elem_t>(xv[i]);
+      for (int i = 0; i < 4; ++i) old[i] = xv[i];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int c = lane + 64 * i;
+        if (c < rh) {
+          const float cs = to_f32(a.cos_t[trow + c]), sn = to_f32(a.sin_t[trow + c]);
+          const float other = in_lane ? (i + shift < 4 ? old[(i + shift) & 3] : 0.f) : y[c + rh];
+          xv[i] = old[i] * cs - other * sn;
+        } else if (c < 2 * rh) {
+          const float cs = to_f32(a.cos_t[trow + c - rh]), sn = to_f32(a.sin_t[trow + c - rh]);
+          const float other = in_lane ? (i >= shift ? old[(i - shift) & 3] : 0.f) : y[c - rh];
+          xv[i] = old[i] * cs + other * sn;
+        }
+      }
     }
-  } else {
-    const int kh = hh - a.nq - a.nkv;
-    elem_t* o = a.vc + ((int64_t)page * a.nkv + kh) * d * a.P + off;
+    if (a.cos_t != nullptr && !in_lane) __syncthreads();    // y is free for the next head
+    if (!live) continue;
+    if (kind == 0) {
+      elem_t* o = a.q_out + ((int64_t)tok * a.nq + hh) * d;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int c = lane + 64 * i;
-      if (c < d) o[(int64_t)c * a.P] = from_f32<elem_t>(xv[i]);
+      for (int i = 0; i < 4; ++i) {
+        const int c = lane + 64 * i;
+        if (c < d) o[c] = from_f32<elem_t>(xv[i]);
+      }
+      continue;
+    }
+    if (slot < 0) continue;
+    const int page = slot / a.P, off = slot - page * a.P;
+    if (kind == 1) {
+      const int kh = hh - a.nq;
+      elem_t* o = a.kc + (((int64_t)page * a.nkv + kh) * a.P + off) * d;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int c = lane + 64 * i;
+        if (c < d) o[c] = from_f32<elem_t>(xv[i]);
+      }
+    } else {
+      const int kh = hh - a.nq - a.nkv;
+      elem_t* o = a.vc + ((int64_t)page * a.nkv + kh) * d * a.P + off;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int c = lane + 64 * i;
+        if (c < d) o[(int64_t)c * a.P] = from_f32<elem_t>(xv[i]);
+      }
     }
   }
 }
@@ -132,7 +154,10 @@ int vk_qkv_post(const elem_t* qkv, int64_t row_stride, elem_t* q_out, elem_t* kc
   a.qkv = qkv; a.row_stride = row_stride; a.q_out = q_out; a.kc = kc; a.vc = vc; a.q_w = q_w; a.k_w = k_w;
   a.cos_t = cos_t; a.sin_t = sin_t; a.positions = positions; a.slots = slots; a.w_is_f32 = w_is_f32;
   a.nq = nq; a.nkv = nkv; a.d = d; a.P = P; a.rot_half = rot_half; a.eps = eps;
-  qkv_post_kernel<<<dim3(T, nq + 2 * nkv), 64, 0, st>>>(a);
+  // Few tokens: four heads per workgroup, for many workgroups; many tokens: all heads of a token.
+  const int heads = nq + 2 * nkv;
+  const int per_wave = T >= 512 ? (heads + 3) / 4 : 1;
+  qkv_post_kernel<<<dim3(T, (heads + 4 * per_wave - 1) / (4 * per_wave)), 256, 0, st>>>(a, per_wave);
   return vk_check_launch("qkv_post");
 }
 
