@@ -531,6 +531,17 @@ __global__ __launch_bounds__(256, 2) void gemm_pipe_kernel(elem_t* __restrict__ 
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[i][j] = mma_slab(wf[i], af[j], acc[i][j]);
     }
+#ifdef VK_BF16
+    // Order for the scheduler: the first slab's reads, then the second slab's reads one by one between
+    // the first slab's MFMAs, so that they return while the matrix unit works.
+    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);     // 8 LDS reads
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);   // 2 MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // 1 LDS read
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, 16, 0);    // the second slab's MFMAs
+#endif
   };
   auto close_chunk = [&]() {
 #pragma unroll
