@@ -382,7 +382,7 @@ __device__ __forceinline__ int val_swz(int row) { return row & 15; }          //
 #endif
 
 template <int DPAD, int QT, int NW>
-__global__ __launch_bounds__(64 * NW) void attn_prefill_lds_kernel(AttnArgs a, int n_items) {
+__global__ __launch_bounds__(64 * NW, 2) void attn_prefill_lds_kernel(AttnArgs a, int n_items) {
   constexpr int ROWS_WG = 16 * QT * NW;                  // NW waves, each with QT 16-row tiles
   constexpr int BPI = ITEM_ROWS / ROWS_WG;               // workgroups per item
   static_assert(ITEM_ROWS % ROWS_WG == 0, "a workgroup's rows must divide an item");
@@ -739,8 +739,8 @@ int vk_attn_segment_keys(void) { return TILE_KEYS * SEG_TILES; }
 
 int vk_attn_item_rows(void) { return ITEM_ROWS; }
 
-// For measurements: 0 is the default shape of the workgroups of the prompt kernel, 14 and 24 are the
-// others (row tiles per wave * 10 + waves).  The result is the same bits.
+// For measurements: 0 is the default shape of the workgroups of the prompt kernel, 14 is the other
+// (row tiles per wave * 10 + waves).  The result is the same bits.
 static int vk_prefill_variant = 0;
 void vk_attn_set_prefill_variant(int v) { vk_prefill_variant = v; }
 
@@ -787,11 +787,13 @@ int vk_paged_attention(elem_t* out, const elem_t* q, const elem_t* kc, const ele
     attn_prefill_lds_kernel<DP, QT, NW><<<n_items * (ITEM_ROWS / (16 * QT * NW)) * nq, 64 * NW, smem, st>>>(a, n_items); \
   } while (0)
     // Eight waves of one row tile each measured best on long contexts (MI355X, head size 128); four
-    // waves are a few per cent better on short ones, two row tiles per wave need too many registers.
+    // waves are a few per cent better on short ones.  Two row tiles per wave (QT = 2) would halve the
+    // LDS traffic but need more than the 256 registers that two waves per SIMD leave: with spills or
+    // with one wave per SIMD they measured 40 % slower.
     const int v = vk_prefill_variant;
-    if (d == 64) { if (v == 14) PREFILL_LDS(64, 1, 4); else if (v == 24) PREFILL_LDS(64, 2, 4); else PREFILL_LDS(64, 1, 8); }
-    else if (d == 128) { if (v == 14) PREFILL_LDS(128, 1, 4); else if (v == 24) PREFILL_LDS(128, 2, 4); else PREFILL_LDS(128, 1, 8); }
-    else { if (v == 14) PREFILL_LDS(256, 1, 4); else if (v == 24) PREFILL_LDS(256, 2, 4); else PREFILL_LDS(256, 1, 8); }
+    if (d == 64) { if (v == 14) PREFILL_LDS(64, 1, 4); else PREFILL_LDS(64, 1, 8); }
+    else if (d == 128) { if (v == 14) PREFILL_LDS(128, 1, 4); else PREFILL_LDS(128, 1, 8); }
+    else { if (v == 14) PREFILL_LDS(256, 1, 4); else PREFILL_LDS(256, 1, 8); }
 #undef PREFILL_LDS
     return vk_check_launch("attention (prompt rows, shared tiles)");
   }
