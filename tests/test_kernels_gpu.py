@@ -351,6 +351,23 @@ def test_attention_prompt_kernels_agree(dtype, nq, nkv, d, P, window):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_many_decoded_tokens(dtype):
+    """Enough decoded tokens and segments (more than a thousand workgroups) that the decode kernel
+    takes its other order of loads: the plain result, and the bits of the same tokens in a small launch."""
+    k = kern(dtype)
+    nq, nkv, d, P = 8, 8, 64, 16
+    lens = [2100 - 83 * i for i in range(24)]
+    q_list = [rand((1, nq, d), dtype, 10 + i) for i in range(24)]
+    kk = [rand((n, nkv, d), dtype, 40 + i) for i, n in enumerate(lens)]
+    vv = [rand((n, nkv, d), dtype, 70 + i) for i, n in enumerate(lens)]
+    got = run_attention(k, q_list, kk, vv, P, dtype, poison=float("nan"))
+    for i in (0, 11, 23):
+        torch.testing.assert_close(got[i:i + 1].float(), plain.attention(q_list[i], kk[i], vv[i], d ** -0.5, dtype), **tol(dtype))
+        alone = run_attention(k, q_list[i:i + 1], kk[i:i + 1], vv[i:i + 1], P, dtype)
+        assert torch.equal(alone[0], got[i])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_attention_far_key_in_prompt_rows(dtype):
     """A key that outweighs all others, seen from the rows of a late portion of a prompt: every row at
     or after it must return its value, through the kernel that shares tiles and the other one.  Then
