@@ -100,7 +100,7 @@ class CacheManager {
     int window;
     int num_pages;
     std::deque<int> free;
-    std::vector<int> holders;   // per page: requests holding it (+1 while it sits in a prefix node)
+    std::vector<int> holders;   // per page, its state: PAGE_FREE (in the free queue), PAGE_PRIVATE (one request's own) or PAGE_NODE (in a prefix node)
   };
   // A published full page per group ("block"): node of the prefix tree.
   struct Node {
