@@ -352,19 +352,29 @@ def test_attention_prompt_kernels_agree(dtype, nq, nkv, d, P, window):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_attention_many_decoded_tokens(dtype):
-    """Enough decoded tokens and segments (more than a thousand workgroups) that the decode kernel
-    takes its other order of loads: the plain result, and the bits of the same tokens in a small launch."""
+    """The decode kernels: keys split over workgroups by segment, with few workgroups (keys and values
+    asked for together) and with more than a thousand (values later), and one workgroup per token and
+    kv head: the plain result and the same bits, with and without a window, for groups of 1 and 20 q heads."""
     k = kern(dtype)
-    nq, nkv, d, P = 8, 8, 64, 16
-    lens = [2100 - 83 * i for i in range(24)]
-    q_list = [rand((1, nq, d), dtype, 10 + i) for i in range(24)]
-    kk = [rand((n, nkv, d), dtype, 40 + i) for i, n in enumerate(lens)]
-    vv = [rand((n, nkv, d), dtype, 70 + i) for i, n in enumerate(lens)]
-    got = run_attention(k, q_list, kk, vv, P, dtype, poison=float("nan"))
-    for i in (0, 11, 23):
-        torch.testing.assert_close(got[i:i + 1].float(), plain.attention(q_list[i], kk[i], vv[i], d ** -0.5, dtype), **tol(dtype))
-        alone = run_attention(k, q_list[i:i + 1], kk[i:i + 1], vv[i:i + 1], P, dtype)
-        assert torch.equal(alone[0], got[i])
+    P = 16
+    for nq, nkv, d, window in ((8, 8, 64, 0), (8, 8, 64, 300), (20, 1, 48, 0)):
+        lens = [2100 - 83 * i for i in range(24)]
+        q_list = [rand((1, nq, d), dtype, 10 + i) for i in range(24)]
+        kk = [rand((n, nkv, d), dtype, 40 + i) for i, n in enumerate(lens)]
+        vv = [rand((n, nkv, d), dtype, 70 + i) for i, n in enumerate(lens)]
+        try:
+            k.lib.vk_attn_set_decode_variant(2)
+            got = run_attention(k, q_list, kk, vv, P, dtype, window=window, poison=float("nan"))
+            k.lib.vk_attn_set_decode_variant(1)
+            whole = run_attention(k, q_list, kk, vv, P, dtype, window=window, poison=float("nan"), seed=4)
+        finally:
+            k.lib.vk_attn_set_decode_variant(0)
+        assert torch.equal(whole, got)
+        for i in (0, 11, 23):
+            ref = plain.attention(q_list[i], kk[i], vv[i], d ** -0.5, dtype, window=window)
+            torch.testing.assert_close(got[i:i + 1].float(), ref, **tol(dtype))
+            alone = run_attention(k, q_list[i:i + 1], kk[i:i + 1], vv[i:i + 1], P, dtype, window=window)
+            assert torch.equal(alone[0], got[i])
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

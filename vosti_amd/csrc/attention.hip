@@ -672,6 +672,98 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
   }
 }
 
+// Decoded tokens, all keys of a token in one workgroup: for batches that fill the chip without a
+// split over segments, and contexts whose tile results fit LDS.  Eight waves take the tiles in turn
+// (wave w: tiles first + w, first + w + 8, ...), every tile's (m, l, acc) goes to LDS, and after one
+// barrier the threads fold them exactly as attn_decode and attn_combine do together: tiles into
+// their segment in order, segments into the total in order.  No scratch buffer, no second launch.
+#define WHOLE_WAVES 8
+template <int DPAD>
+__global__ __launch_bounds__(64 * WHOLE_WAVES) void attn_decode_whole_kernel(AttnArgs a, int tiles_cap) {
+  constexpr int NDT = DPAD / 16, NQS = DPAD / VK_SLAB;
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int G = a.nq / a.nkv, HT = (G + 15) >> 4;
+  const int kvh = blockIdx.y / HT, ht = blockIdx.y - kvh * HT;
+  const int nvalid = min(16, G - ht * 16);
+  float* s_acc = smem;                                         // [tiles_cap][nvalid][DPAD]
+  float* s_ml = smem + (size_t)tiles_cap * nvalid * DPAD;      // [tiles_cap][nvalid][2]
+  const int seq = a.items[2 * blockIdx.x], q_off = a.items[2 * blockIdx.x + 1];
+  const int q_begin = a.cu_q[seq], q_len = a.cu_q[seq + 1] - q_begin;
+  const int k_len = a.k_len[seq];
+  const int tok = q_begin + q_off;
+  const int pos = k_len - q_len + q_off;
+  const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+  const int tile_lo = lo / TILE_KEYS, tile_hi = pos / TILE_KEYS;   // tile_hi - tile_lo < tiles_cap (host)
+
+  RowCtx c;
+  init_ctx(c, a, seq, kvh, k_len);
+  c.r16 = lane & 15;
+  c.g = lane >> 4;
+  c.row_ok = c.r16 < nvalid;
+  c.pos = pos;
+  c.lo = lo;
+  c.wave_lo = lo;
+  const int head0 = kvh * G + ht * 16;
+  frag_t qf[NQS];
+  load_q<NQS>(a, tok, head0 + c.r16, c.row_ok, c.g, qf);
+  for (int t = tile_lo + wave; t <= tile_hi; t += WHOLE_WAVES) {
+    float m_t, l_t;
+    f32x4 acc[NDT];
+    tile_partial<NDT, NQS, false>(c, qf, t * TILE_KEYS, m_t, l_t, acc);
+    if (c.row_ok) {
+      float* dst = s_acc + ((size_t)(t - tile_lo) * nvalid + c.r16) * DPAD;
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt)
+        if (dt * 16 < a.d) *reinterpret_cast<f32x4*>(dst + dt * 16 + 4 * c.g) = acc[dt];
+      if (c.g == 0) {
+        s_ml[((t - tile_lo) * nvalid + c.r16) * 2] = m_t;
+        s_ml[((t - tile_lo) * nvalid + c.r16) * 2 + 1] = l_t;
+      }
+    }
+  }
+  __syncthreads();
+  // Thread (row, column group) owns DPAD/16 columns of one row.
+  const int row = threadIdx.x >> 4, cg = threadIdx.x & 15;
+  if (row >= nvalid) return;
+  float M = -INFINITY, L = 0.f;
+  float ACC[NDT];
+#pragma unroll
+  for (int i = 0; i < NDT; ++i) ACC[i] = 0.f;
+  for (int seg = tile_lo / SEG_TILES; seg <= tile_hi / SEG_TILES; ++seg) {
+    float Ms = -INFINITY, Ls = 0.f;
+    float As[NDT];
+#pragma unroll
+    for (int i = 0; i < NDT; ++i) As[i] = 0.f;
+    const int t_end = min(tile_hi, seg * SEG_TILES + SEG_TILES - 1);
+    for (int t = max(tile_lo, seg * SEG_TILES); t <= t_end; ++t) {
+      const int e = (t - tile_lo) * nvalid + row;
+      const float m = s_ml[2 * e], l = s_ml[2 * e + 1];
+      if (m > -INFINITY) {
+        float Mn, ca, cb;
+        fold_scales(Ms, m, Mn, ca, cb);
+#pragma unroll
+        for (int i = 0; i < NDT; ++i) As[i] = fold1(As[i], s_acc[(size_t)e * DPAD + cg * NDT + i], ca, cb);
+        Ls = fold1(Ls, l, ca, cb);
+        Ms = Mn;
+      }
+    }
+    if (Ms > -INFINITY) {
+      float Mn, ca, cb;
+      fold_scales(M, Ms, Mn, ca, cb);
+#pragma unroll
+      for (int i = 0; i < NDT; ++i) ACC[i] = fold1(ACC[i], As[i], ca, cb);
+      L = fold1(L, Ls, ca, cb);
+      M = Mn;
+    }
+  }
+  const float inv = L > 0.f ? 1.0f / L : 0.f;
+  elem_t* orow = a.out + ((int64_t)tok * a.nq + head0 + row) * a.d;
+#pragma unroll
+  for (int i = 0; i < NDT; ++i)
+    if (cg * NDT + i < a.d) orow[cg * NDT + i] = from_f32<elem_t>(ACC[i] * inv);
+}
+
 // Folds the segment results of one (token, head) in ascending segment order.
 // One wave per row; lane j owns output columns j, j+64, ...
 __global__ __launch_bounds__(64) void attn_combine_kernel(AttnArgs a) {
@@ -743,6 +835,11 @@ int vk_attn_item_rows(void) { return ITEM_ROWS; }
 // (row tiles per wave * 10 + waves).  The result is the same bits.
 static int vk_prefill_variant = 0;
 void vk_attn_set_prefill_variant(int v) { vk_prefill_variant = v; }
+// 0: the decode kernel is chosen by size, 1: one workgroup per token and kv head where LDS allows,
+// 2: always the split over segments.  The result is the same bits.
+static int vk_decode_variant = 0;
+void vk_attn_set_decode_variant(int v) { vk_decode_variant = v; }
+static int vk_dpad(int d) { return d <= 64 ? 64 : (d <= 128 ? 128 : 256); }
 
 // 1 if prompt rows of this shape go through the kernel that shares key tiles in LDS.
 int vk_attn_prefill_shares_tiles(int d, int P) {
@@ -808,6 +905,36 @@ int vk_paged_attention(elem_t* out, const elem_t* q, const elem_t* kc, const ele
     return vk_check_launch("attention (prompt rows)");
   }
   VK_REQUIRE(nseg > 0 && nseg <= 65535 && scratch != nullptr, "attention: decode needs nseg in 1..65535 and scratch");
+  {
+    // One workgroup per (token, kv head) when there are enough of them to fill the chip's memory pipes
+    // and the tiles' results fit LDS; else the keys are split over workgroups by segment (below).
+    // Measured on MI355X at 2,060 keys and head size 128: 64 tokens 110 against 117 us, 16 tokens 45
+    // against 35 us (a wave walks its tiles one after the other, so few workgroups are latency-bound).
+    const int HT = (G + 15) / 16, rows = G < 16 ? G : 16;
+    const int tiles_cap = nseg * SEG_TILES;
+    const size_t smem = (size_t)tiles_cap * rows * (vk_dpad(d) + 2) * sizeof(float);
+    const int64_t wgs = (int64_t)n_items * nkv * HT;
+    const bool whole = vk_decode_variant == 1 || (vk_decode_variant == 0 && wgs >= 448 && smem <= 96 * 1024);
+    if (whole && smem <= 150 * 1024) {
+      const dim3 grid(n_items, nkv * HT);
+      VK_REQUIRE(grid.y <= 65535, "attention: too many heads");
+#define DECODE_WHOLE(DP)                                                                             \
+  do {                                                                                               \
+    static bool raised = false;                                                                      \
+    if (!raised) {                                                                                   \
+      (void)hipFuncSetAttribute((const void*)attn_decode_whole_kernel<DP>,                           \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);             \
+      raised = true;                                                                                 \
+    }                                                                                                \
+    attn_decode_whole_kernel<DP><<<grid, 64 * WHOLE_WAVES, smem, st>>>(a, tiles_cap);                \
+  } while (0)
+      if (d <= 64) DECODE_WHOLE(64);
+      else if (d <= 128) DECODE_WHOLE(128);
+      else DECODE_WHOLE(256);
+#undef DECODE_WHOLE
+      return vk_check_launch("attention (decoded rows, whole)");
+    }
+  }
   a.part_ml = scratch;
   a.part_acc = scratch + (((int64_t)total_tokens * nq * nseg * 2 + 3) & ~(int64_t)3);
   const dim3 grid(n_items, nkv * ((G + 15) / 16), nseg);
