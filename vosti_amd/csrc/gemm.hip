@@ -463,7 +463,12 @@ __device__ __forceinline__ void wait_vmcnt(int n) {
   }
 }
 
-template <int S, bool WHOLE>
+// With SWIGLU the weight holds N gate rows, then N up rows, and the output has N columns: a workgroup
+// takes 64 gate rows and the matching 64 up rows as its 128 weight rows (the waves with wn = 0 the
+// gate, those with wn = 1 the up projection), and at the end the up values pass through LDS to the
+// waves that hold the gate values, which write  silu(g) * u  with g and u rounded to the element type
+// first: the bits of the plain projection followed by swiglu_kernel.
+template <int S, bool WHOLE, bool SWIGLU>
 __global__ __launch_bounds__(256, 2) void gemm_pipe_kernel(elem_t* __restrict__ out, const elem_t* __restrict__ act,
                                                         const elem_t* __restrict__ w, int M, int N, int K,
                                                         int64_t lda, int64_t ldo, int out_vec_ok) {
@@ -473,7 +478,7 @@ __global__ __launch_bounds__(256, 2) void gemm_pipe_kernel(elem_t* __restrict__ 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r16 = lane & 15, kg = lane >> 4;
   const int wn = wave & 1, wm = wave >> 1;
-  const int n_blk = blockIdx.x * 128, m_blk = blockIdx.y * 128;
+  const int n_blk = blockIdx.x * (SWIGLU ? 64 : 128), m_blk = blockIdx.y * 128;
   const int ntiles = K / (2 * VK_SLAB);
 
   // A wave-level load moves 8 rows x 128 bytes; lane i fills LDS slot i of the 1 KB block, which is
@@ -484,7 +489,8 @@ __global__ __launch_bounds__(256, 2) void gemm_pipe_kernel(elem_t* __restrict__ 
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int row = (wave * 4 + j) * 8 + lr;
-    gw[j] = w + (int64_t)min(n_blk + row, N - 1) * K + lc * VK_VEC;
+    const int wrow = SWIGLU ? (row < 64 ? min(n_blk + row, N - 1) : N + min(n_blk + row - 64, N - 1)) : min(n_blk + row, N - 1);
+    gw[j] = w + (int64_t)wrow * K + lc * VK_VEC;
     ga[j] = act + (int64_t)min(m_blk + row, M - 1) * lda + lc * VK_VEC;
   }
   auto issue = [&](int kt) {
@@ -570,6 +576,37 @@ __global__ __launch_bounds__(256, 2) void gemm_pipe_kernel(elem_t* __restrict__ 
     }
   }
 
+  if (SWIGLU) {
+    // The two waves of a row block split the 64 output columns: the gate wave keeps columns 0..31 and
+    // gets their up values, the up wave keeps columns 32..63 and gets their gate values.
+    __syncthreads();            // the last tile has been read: LDS is free
+    f32x4* ex = reinterpret_cast<f32x4*>(lds);      // [128 rows][16 groups of 4 columns]
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        f32x4& v = total[i][j];
+        v.x = round_to_elem(v.x); v.y = round_to_elem(v.y); v.z = round_to_elem(v.z); v.w = round_to_elem(v.w);
+        if ((i < 2) == (wn == 1)) ex[(wm * 64 + j * 16 + r16) * 16 + i * 4 + kg] = v;    // what the other wave needs
+      }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if ((i < 2) != (wn == 0)) continue;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const f32x4 o = ex[(wm * 64 + j * 16 + r16) * 16 + i * 4 + kg];
+        const f32x4 g = wn == 0 ? total[i][j] : o, u = wn == 0 ? o : total[i][j];
+        f32x4 y;
+        y.x = (g.x * (1.0f / (1.0f + expf(-g.x)))) * u.x;
+        y.y = (g.y * (1.0f / (1.0f + expf(-g.y)))) * u.y;
+        y.z = (g.z * (1.0f / (1.0f + expf(-g.z)))) * u.z;
+        y.w = (g.w * (1.0f / (1.0f + expf(-g.w)))) * u.w;
+        store_out4(out, ldo, m_blk + wm * 64 + j * 16 + r16, n_blk + i * 16 + 4 * kg, M, N, y, out_vec_ok);
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -578,20 +615,20 @@ __global__ __launch_bounds__(256, 2) void gemm_pipe_kernel(elem_t* __restrict__ 
                  out_vec_ok);
 }
 
-template <int S>
+template <int S, bool SWIGLU = false>
 static int launch_pipe(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K, int64_t lda, int64_t ldo,
                        int vec_ok, hipStream_t st) {
-  const size_t smem = (size_t)S * 2 * 128 * T_ROWB;
+  const size_t smem = (size_t)S * 2 * 128 * T_ROWB;     // also holds the 32 KB that SWIGLU passes between waves
   static bool configured = false;
   if (!configured) {
-    (void)hipFuncSetAttribute((const void*)gemm_pipe_kernel<S, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    (void)hipFuncSetAttribute((const void*)gemm_pipe_kernel<S, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    (void)hipFuncSetAttribute((const void*)gemm_pipe_kernel<S, true, SWIGLU>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    (void)hipFuncSetAttribute((const void*)gemm_pipe_kernel<S, false, SWIGLU>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     configured = true;
   }
-  dim3 grid((N + 127) / 128, (M + 127) / 128);
+  dim3 grid((N + (SWIGLU ? 63 : 127)) / (SWIGLU ? 64 : 128), (M + 127) / 128);
   VK_REQUIRE(grid.y <= 65535, "gemm: too many rows (%d)", M);
-  if (K % KC == 0) gemm_pipe_kernel<S, true><<<grid, 256, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok);
-  else gemm_pipe_kernel<S, false><<<grid, 256, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok);
+  if (K % KC == 0) gemm_pipe_kernel<S, true, SWIGLU><<<grid, 256, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok);
+  else gemm_pipe_kernel<S, false, SWIGLU><<<grid, 256, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok);
   return vk_check_launch("gemm_pipe");
 }
 
@@ -668,14 +705,22 @@ int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K
 }
 
 // 1 if vk_gemm_swiglu takes these sizes (the caller otherwise runs vk_gemm and vk_swiglu, with the same result).
-int vk_gemm_swiglu_supported(int M, int I, int K) { return M >= 1 && M <= 16 && I > 0 && K % KC == 0 && K <= SK_WAVES * KC; }
+// 1: the streaming kernel (few rows), 2: the pipelined tile kernel (many rows), 0: neither.
+int vk_gemm_swiglu_supported(int M, int I, int K) {
+  if (M >= 1 && M <= 16 && I > 0 && K % KC == 0 && K <= SK_WAVES * KC) return 1;
+  if (M > 64 && I > 0 && K % (2 * VK_SLAB) == 0) return 2;
+  return 0;
+}
 
 // out[M, I] = silu(act w_gate^T) * (act w_up^T), w = [gate rows; up rows] of shape [2I, K].
 int vk_gemm_swiglu(elem_t* out, const elem_t* act, const elem_t* w, int M, int I, int K, int64_t lda, int64_t ldo,
                    hipStream_t st) {
-  VK_REQUIRE(vk_gemm_swiglu_supported(M, I, K), "gemm_swiglu: sizes M=%d I=%d K=%d are not supported", M, I, K);
+  const int how = vk_gemm_swiglu_supported(M, I, K);
+  VK_REQUIRE(how != 0, "gemm_swiglu: sizes M=%d I=%d K=%d are not supported", M, I, K);
   VK_REQUIRE(lda >= K && lda % VK_VEC == 0 && ldo >= I, "gemm_swiglu: bad row strides");
   VK_REQUIRE(((uintptr_t)act % 16) == 0 && ((uintptr_t)w % 16) == 0, "gemm_swiglu: operands must be 16-byte aligned");
+  if (how == 2)
+    return launch_pipe<2, true>(out, act, w, M, I, K, lda, ldo, (ldo % 4 == 0) && ((uintptr_t)out % 16 == 0), st);
   static int resident = 0;
   if (resident == 0) {
     int dev = 0, cus = 0, per_cu = 0;
