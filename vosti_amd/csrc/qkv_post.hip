@@ -131,6 +131,79 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvPostArgs a, int per_wa
   }
 }
 
+// The same for head sizes 64, 128 and 256 with a full rotation (or none): a lane owns VK_VEC
+// consecutive elements, so that rows are read and written 16 bytes per lane; the d / VK_VEC lanes of a
+// head sit side by side, a wave holds 64 / (d / VK_VEC) heads of one token.  The sum of squares runs
+// over a lane's elements in order, then as a butterfly over the head's lanes.
+template <int LPH>     // lanes per head
+__global__ __launch_bounds__(256) void qkv_post_vec_kernel(QkvPostArgs a, int per_wave) {
+  constexpr int HPW = 64 / LPH;
+  const int tok = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int d = a.d, heads = a.nq + 2 * a.nkv;
+  const int j = lane % LPH, hsub = lane / LPH;
+  int64_t trow = 0;
+  if (a.cos_t != nullptr) trow = (int64_t)a.positions[tok] * a.rot_half;
+  const int slot = a.slots != nullptr ? a.slots[tok] : -1;
+  const int page = slot >= 0 ? slot / a.P : 0, off = slot >= 0 ? slot - page * a.P : 0;
+  for (int it = 0; it < per_wave; ++it) {
+    const int hh = ((blockIdx.y * per_wave + it) * 4 + wave) * HPW + hsub;
+    const bool live = hh < heads;
+    const int kind = hh < a.nq ? 0 : (hh < a.nq + a.nkv ? 1 : 2);   // q, k, v
+    const elem_t* x = a.qkv + tok * a.row_stride + (int64_t)(live ? hh : 0) * d + j * VK_VEC;
+    const void* w = kind == 0 ? a.q_w : (kind == 1 ? a.k_w : nullptr);
+    float xv[VK_VEC];
+    load_elems(x, xv);
+    if (w != nullptr) {
+      float part = 0.f;
+#pragma unroll
+      for (int e = 0; e < VK_VEC; ++e) part = part + xv[e] * xv[e];
+#pragma unroll
+      for (int m = 1; m < LPH; m <<= 1) part = part + __shfl_xor(part, m, VK_WAVE);
+      const float rr = rsqrtf(part / (float)d + a.eps);
+      float wv[VK_VEC];
+      if (a.w_is_f32) {
+#pragma unroll
+        for (int e = 0; e < VK_VEC; ++e) wv[e] = static_cast<const float*>(w)[j * VK_VEC + e];
+      } else {
+        load_elems(static_cast<const elem_t*>(w) + j * VK_VEC, wv);
+      }
+#pragma unroll
+      for (int e = 0; e < VK_VEC; ++e) xv[e] = round_to_elem((xv[e] * rr) * wv[e]);
+    }
+    if (a.cos_t != nullptr) {
+      // The partner of element c is c +- d/2: the same place in the lane LPH/2 away.  Every lane takes
+      // part in the exchange, also those of v heads, which keep their values.
+      float other[VK_VEC], cs[VK_VEC], sn[VK_VEC];
+#pragma unroll
+      for (int e = 0; e < VK_VEC; ++e) other[e] = __shfl_xor(xv[e], LPH / 2, VK_WAVE);
+      const int tcol = (j % (LPH / 2)) * VK_VEC;
+      load_elems(a.cos_t + trow + tcol, cs);
+      load_elems(a.sin_t + trow + tcol, sn);
+      if (kind != 2) {
+        if (j < LPH / 2) {
+#pragma unroll
+          for (int e = 0; e < VK_VEC; ++e) xv[e] = xv[e] * cs[e] - other[e] * sn[e];
+        } else {
+#pragma unroll
+          for (int e = 0; e < VK_VEC; ++e) xv[e] = xv[e] * cs[e] + other[e] * sn[e];
+        }
+      }
+    }
+    if (!live) continue;
+    if (kind == 0) {
+      store_elems(a.q_out + ((int64_t)tok * a.nq + hh) * d + j * VK_VEC, xv);
+    } else if (slot >= 0) {
+      if (kind == 1) {
+        store_elems(a.kc + (((int64_t)page * a.nkv + (hh - a.nq)) * a.P + off) * d + j * VK_VEC, xv);
+      } else {
+        elem_t* o = a.vc + (((int64_t)page * a.nkv + (hh - a.nq - a.nkv)) * d + j * VK_VEC) * a.P + off;
+#pragma unroll
+        for (int e = 0; e < VK_VEC; ++e) o[(int64_t)e * a.P] = from_f32<elem_t>(xv[e]);
+      }
+    }
+  }
+}
+
 extern "C" {
 
 // Null q_w / k_w: no norm for that kind.  Null cos_t: no rotation.  nkv == 0:
@@ -154,8 +227,22 @@ int vk_qkv_post(const elem_t* qkv, int64_t row_stride, elem_t* q_out, elem_t* kc
   a.qkv = qkv; a.row_stride = row_stride; a.q_out = q_out; a.kc = kc; a.vc = vc; a.q_w = q_w; a.k_w = k_w;
   a.cos_t = cos_t; a.sin_t = sin_t; a.positions = positions; a.slots = slots; a.w_is_f32 = w_is_f32;
   a.nq = nq; a.nkv = nkv; a.d = d; a.P = P; a.rot_half = rot_half; a.eps = eps;
-  // Few tokens: four heads per workgroup, for many workgroups; many tokens: all heads of a token.
+  // Few tokens: four waves' worth of heads per workgroup, for many workgroups; many tokens: all heads of a token.
   const int heads = nq + 2 * nkv;
+  const int lph = d / VK_VEC;          // lanes per head in the kernel with 16-byte accesses
+  const bool vec = (d == 64 || d == 128 || d == 256) && lph <= 64 && (cos_t == nullptr || 2 * rot_half == d) &&
+                   row_stride % VK_VEC == 0 && ((uintptr_t)qkv % 16) == 0 && (q_out == nullptr || (uintptr_t)q_out % 16 == 0) &&
+                   (kc == nullptr || (uintptr_t)kc % 16 == 0) && (cos_t == nullptr || ((uintptr_t)cos_t % 16 == 0 && (uintptr_t)sin_t % 16 == 0));
+  if (vec) {
+    const int hpw = 64 / lph, per_wg = 4 * hpw;
+    const int per_wave = T >= 512 ? (heads + per_wg - 1) / per_wg : 1;
+    const dim3 grid(T, (heads + per_wg * per_wave - 1) / (per_wg * per_wave));
+    if (lph == 8) qkv_post_vec_kernel<8><<<grid, 256, 0, st>>>(a, per_wave);
+    else if (lph == 16) qkv_post_vec_kernel<16><<<grid, 256, 0, st>>>(a, per_wave);
+    else if (lph == 32) qkv_post_vec_kernel<32><<<grid, 256, 0, st>>>(a, per_wave);
+    else qkv_post_vec_kernel<64><<<grid, 256, 0, st>>>(a, per_wave);
+    return vk_check_launch("qkv_post");
+  }
   const int per_wave = T >= 512 ? (heads + 3) / 4 : 1;
   qkv_post_kernel<<<dim3(T, (heads + 4 * per_wave - 1) / (4 * per_wave)), 256, 0, st>>>(a, per_wave);
   return vk_check_launch("qkv_post");
