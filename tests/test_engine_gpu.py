@@ -184,6 +184,19 @@ def test_command_line(tiny_dirs, tmp_path, dtype_name):
     assert r.returncode == 0, r.stderr[-2000:]
     assert "BENCH batch=2 prompt_tokens=5 output_tokens=7" in r.stdout
     assert [len(l.split("\t")[1].split(",")) for l in (tmp_path / "o2.tsv").read_text().splitlines()] == [3, 4]
+    # A warm-up workload in the same engine first (examples/support/engine_serving.rs:157-206); the measured
+    # requests then find the page that the warm-up left: 16 tokens of the 20 they share.
+    shared = ",".join(str(7 + (i * 5) % 200) for i in range(20))
+    (tmp_path / "warm.tsv").write_text(f"2\t{shared},5\n")
+    (tmp_path / "meas.tsv").write_text(f"2\t{shared},9\n2\t{shared},11,12\n")
+    env3 = dict(env, VOSTI_BENCH_INPUT=str(tmp_path / "meas.tsv"), VOSTI_BENCH_WARMUP_INPUT=str(tmp_path / "warm.tsv"),
+                VOSTI_NUM_BLOCKS="12", VOSTI_PAGE_SIZE="16", VOSTI_MAX_MODEL_LEN="64")
+    r = subprocess.run([sys.executable, "-m", "vosti_amd.launch", "--kind", "engine", "--family", "qwen3"], env=env3,
+                       capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert "WARMUP batch=1 prompt_tokens=21 output_tokens=2" in r.stdout
+    assert 'WARMUP_CACHE_STATS {"admitted_requests":1,"requests_with_reuse":0,"reused_prefix_blocks":0}' in r.stdout
+    assert 'CACHE_STATS {"admitted_requests":2,"requests_with_reuse":2,"reused_prefix_blocks":2' in r.stdout
 
 
 def test_smoke_entry():

@@ -6,7 +6,7 @@ from ctypes import POINTER, c_char_p, c_int, c_int32, c_int64, c_uint64, c_void_
 
 from ..kernels import build
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 _LIB = None
 
 
@@ -38,6 +38,7 @@ def host_lib():
     for n in ("free_slots", "num_requests", "cached_blocks"):
         sig(f"vh_cache_{n}", I, P)
     sig("vh_cache_prefix_hits", c_int64, P)
+    sig("vh_cache_prefix_hit_requests", c_int64, P)
     sig("vh_cache_evictions", c_int64, P)
     sig("vh_cache_fill_block_table", I, P, U, I, c_void_p, I)
     sig("vh_cache_fill_slots", I, P, U, I, I, I, c_void_p)

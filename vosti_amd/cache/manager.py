@@ -134,6 +134,10 @@ class CacheManager:
     def prefix_hits(self) -> int:
         return self._lib.vh_cache_prefix_hits(self._h)
 
+    def prefix_hit_requests(self) -> int:
+        """Admissions that found at least one cached page."""
+        return self._lib.vh_cache_prefix_hit_requests(self._h)
+
     def evictions(self) -> int:
         return self._lib.vh_cache_evictions(self._h)
 

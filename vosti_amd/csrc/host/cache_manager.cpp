@@ -143,6 +143,7 @@ Status CacheManager::add_request(RequestId id, const int32_t* prompt, int n_prom
     r.length = r.published * page_size_;
     r.tokens.assign(prompt, prompt + r.length);
     prefix_hit_pages_ += r.published;
+    if (r.published > 0) ++prefix_hit_requests_;
     if (cached_tokens) *cached_tokens = r.length;
   }
   requests_.emplace(id, std::move(r));

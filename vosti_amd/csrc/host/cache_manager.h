@@ -88,6 +88,7 @@ class CacheManager {
 
   // Counters for tests and logs.
   int64_t prefix_hits() const { return prefix_hit_pages_; }
+  int64_t prefix_hit_requests() const { return prefix_hit_requests_; }   // admissions that found a cached prefix
   int64_t evictions() const { return evictions_; }
   int cached_blocks() const { return (int)lru_.size(); }
 
@@ -147,6 +148,7 @@ class CacheManager {
   std::unordered_map<uint64_t, int> by_hash_;
   std::list<int> lru_;   // cached (refcount 0) nodes, eviction from the front
   int64_t prefix_hit_pages_ = 0;
+  int64_t prefix_hit_requests_ = 0;
   int64_t evictions_ = 0;
 };
 

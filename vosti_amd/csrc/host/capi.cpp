@@ -20,7 +20,7 @@ struct SchedulerHandle {
 
 extern "C" {
 
-int vh_abi_version(void) { return 3; }
+int vh_abi_version(void) { return 4; }
 
 // ------------------------------------------------------------ cache manager
 void* vh_cache_create(int page_size, int n_groups, const int* windows, const int* num_pages, int num_slots,
@@ -55,6 +55,7 @@ int vh_cache_free_slots(void* h) { return CM->free_slots(); }
 int vh_cache_num_requests(void* h) { return CM->num_requests(); }
 int vh_cache_cached_blocks(void* h) { return CM->cached_blocks(); }
 int64_t vh_cache_prefix_hits(void* h) { return CM->prefix_hits(); }
+int64_t vh_cache_prefix_hit_requests(void* h) { return CM->prefix_hit_requests(); }
 int64_t vh_cache_evictions(void* h) { return CM->evictions(); }
 int vh_cache_fill_block_table(void* h, uint64_t id, int g, int32_t* out, int width) {
   return CM->fill_block_table(id, g, out, width);

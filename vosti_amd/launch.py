@@ -20,6 +20,8 @@ here; each also has a command-line option, which wins:
     VOSTI_CUDA_GRAPH           --graphs              0/1: replay decode steps from captured HIP graphs
     VOSTI_OUTPUT_TOKENS        --output-tokens       write "index<TAB>ids" lines to this file
     VOSTI_BENCH_INPUT          --bench-input         TSV of MAX_TOKENS<TAB>IDS[<TAB>ARRIVAL_STEP] requests
+    VOSTI_BENCH_WARMUP_INPUT   --bench-warmup-input  a TSV of other requests, served first by the same engine
+    VOSTI_MAX_MODEL_LEN        --max-model-len       longest prompt plus output (default: the model's positions)
     VOSTI_ENGINE_STEP_TRACE    --step-trace          append one JSON line per step to this file
 
 Options without a counterpart in the reference: VOSTI_DTYPE / --dtype (bfloat16,
@@ -60,6 +62,8 @@ def engine_parser() -> argparse.ArgumentParser:
     p.add_argument("--graphs", type=int, default=int(_env("VOSTI_CUDA_GRAPH", 0)), choices=[0, 1])
     p.add_argument("--output-tokens", default=_env("VOSTI_OUTPUT_TOKENS"))
     p.add_argument("--bench-input", default=_env("VOSTI_BENCH_INPUT"))
+    p.add_argument("--bench-warmup-input", default=_env("VOSTI_BENCH_WARMUP_INPUT"))
+    p.add_argument("--max-model-len", type=int, default=int(_env("VOSTI_MAX_MODEL_LEN", 0)))
     p.add_argument("--step-trace", default=_env("VOSTI_ENGINE_STEP_TRACE"))
     p.add_argument("--dtype", default=_env("VOSTI_DTYPE", "bfloat16"), choices=["bfloat16", "float32"])
     p.add_argument("--temperature", type=float, default=float(_env("VOSTI_TEMPERATURE", 0.0)))
@@ -124,28 +128,48 @@ def run_engine(argv: list[str], family: str) -> int:
         requests = parse_prepared(args.bench_input)
     else:
         requests = [(args.max_tokens, parse_ids(args.prompt_ids), 0)]
+    warmup = parse_prepared(args.bench_warmup_input) if args.bench_input and args.bench_warmup_input else []
     eos = eos_ids(args.model_path)
     engine = Engine(args.model_path, dtype=args.dtype, num_pages=args.num_blocks, page_size=args.page_size,
-                    max_num_seqs=args.max_seqs or len(requests), max_num_batched_tokens=args.max_batched_tokens,
-                    enable_prefix_cache=bool(args.prefix_cache), graphs=bool(args.graphs))
-    params = [SamplingParams(max_tokens=m, temperature=args.temperature, seed=args.seed + i, eos_token_ids=eos,
-                             ignore_eos=args.ignore_eos) for i, (m, _, _) in enumerate(requests)]
+                    max_num_seqs=args.max_seqs or max(len(requests), len(warmup)),
+                    max_num_batched_tokens=args.max_batched_tokens, enable_prefix_cache=bool(args.prefix_cache),
+                    max_model_len=args.max_model_len or None, graphs=bool(args.graphs))
     trace = open(args.step_trace, "a") if args.step_trace else None
     import torch
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    outputs = engine.generate([ids for _, ids, _ in requests], params, [a for _, _, a in requests], trace=trace)
-    wall = time.perf_counter() - t0
+
+    def serve(reqs, first_seed):
+        """(outputs, wall seconds, cache statistics of this workload alone)."""
+        params = [SamplingParams(max_tokens=m, temperature=args.temperature, seed=first_seed + i, eos_token_ids=eos,
+                                 ignore_eos=args.ignore_eos) for i, (m, _, _) in enumerate(reqs)]
+        before = (engine.cache.prefix_hit_requests(), engine.cache.prefix_hits())
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        outs = engine.generate([ids for _, ids, _ in reqs], params, [a for _, _, a in reqs], trace=trace)
+        wall = time.perf_counter() - t0
+        stats = {"admitted_requests": len(reqs), "requests_with_reuse": engine.cache.prefix_hit_requests() - before[0],
+                 "reused_prefix_blocks": engine.cache.prefix_hits() - before[1]}
+        return outs, wall, stats
+
+    def line(tag, reqs, outs, wall, rate):
+        n_out = sum(len(o) for o in outs)
+        text = f"{tag} batch={len(reqs)} prompt_tokens={sum(len(i) for _, i, _ in reqs)} output_tokens={n_out} wall_s={wall:.9f}"
+        return text + (f" tok_s={n_out / wall:.6f}" if rate else "")
+
+    if warmup:
+        # The reference serves a disjoint warm-up workload in the same engine before the measured one
+        # (examples/support/engine_serving.rs:157-206) and reports both (engine_benchmark.rs:45-76).
+        w_out, w_wall, w_stats = serve(warmup, args.seed + len(requests))
+        print(line("WARMUP", warmup, w_out, w_wall, rate=False))
+        print("WARMUP_CACHE_STATS " + json.dumps(w_stats, separators=(",", ":")))
+    outputs, wall, stats = serve(requests, args.seed)
     if trace:
         trace.close()
     if args.output_tokens:
         Path(args.output_tokens).write_text("".join(f"{i}\t{','.join(map(str, o))}\n" for i, o in enumerate(outputs)))
     if args.bench_input:
-        n_out = sum(len(o) for o in outputs)
-        print(f"BENCH batch={len(requests)} prompt_tokens={sum(len(i) for _, i, _ in requests)} output_tokens={n_out} "
-              f"wall_s={wall:.9f} tok_s={n_out / wall:.6f}")
-        print("CACHE_STATS " + json.dumps({"admitted_requests": len(requests), "reused_prefix_blocks": engine.cache.prefix_hits(),
-                                           "preemptions": engine.scheduler.preemptions()}, separators=(",", ":")))
+        print(line("BENCH", requests, outputs, wall, rate=True))
+        stats["preemptions"] = engine.scheduler.preemptions()
+        print("CACHE_STATS " + json.dumps(stats, separators=(",", ":")))
     else:
         print(f"MODEL_OUTPUT_TOKEN_IDS={outputs[0]}")
     if args.graphs:
