@@ -199,6 +199,21 @@ def test_command_line(tiny_dirs, tmp_path, dtype_name):
     assert 'CACHE_STATS {"admitted_requests":2,"requests_with_reuse":2,"reused_prefix_blocks":2' in r.stdout
 
 
+def test_logits_digest(tiny_dirs, tmp_path, monkeypatch):
+    """VOSTI_LOGITS_DIGEST: the hash of every sampled row; a request's hashes are the same alone and in a batch."""
+    from vosti_amd.sampling import SamplingParams
+    ps = prompts("B", [11, 30], seed=5)
+    sp = SamplingParams(max_tokens=4)
+    monkeypatch.setenv("VOSTI_LOGITS_DIGEST", str(tmp_path / "alone.txt"))
+    engine(tiny_dirs["B"], "bfloat16", num_pages=16, page_size=8).generate([ps[1]], sp)
+    monkeypatch.setenv("VOSTI_LOGITS_DIGEST", str(tmp_path / "both.txt"))
+    engine(tiny_dirs["B"], "bfloat16", num_pages=16, page_size=8).generate(ps, sp)
+    alone = [l.split() for l in (tmp_path / "alone.txt").read_text().splitlines()]
+    both = [l.split() for l in (tmp_path / "both.txt").read_text().splitlines()]
+    assert len(alone) == 4 and len(both) == 8 and all(len(h) == 64 for _, h in both)
+    assert [h for i, h in both if i == "1"] == [h for _, h in alone]
+
+
 def test_smoke_entry():
     sys.path.insert(0, str(ROOT))
     import __graft_entry__

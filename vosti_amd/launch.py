@@ -22,6 +22,7 @@ here; each also has a command-line option, which wins:
     VOSTI_BENCH_INPUT          --bench-input         TSV of MAX_TOKENS<TAB>IDS[<TAB>ARRIVAL_STEP] requests
     VOSTI_BENCH_WARMUP_INPUT   --bench-warmup-input  a TSV of other requests, served first by the same engine
     VOSTI_MAX_MODEL_LEN        --max-model-len       longest prompt plus output (default: the model's positions)
+    VOSTI_LOGITS_DIGEST                              a file that gets "row sha256" for every sampled logits row
     VOSTI_ENGINE_STEP_TRACE    --step-trace          append one JSON line per step to this file
 
 Options without a counterpart in the reference: VOSTI_DTYPE / --dtype (bfloat16,
