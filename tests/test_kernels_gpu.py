@@ -378,6 +378,26 @@ def test_attention_many_decoded_tokens(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_long_context(dtype):
+    """20,000 keys: the last 130 rows as a prompt portion and the last row as a decoded token, against
+    the plain result; and a key that outweighs all others at the start, the middle and the end."""
+    k = kern(dtype)
+    nq, nkv, d, P, L, n = 4, 1, 128, 64, 20000, 130
+    q, kx, vx = rand((n, nq, d), dtype, 1), rand((L, nkv, d), dtype, 2), rand((L, nkv, d), dtype, 3)
+    got = run_attention(k, [q], [kx], [vx], P, dtype)
+    ref = plain.attention(q, kx, vx, d ** -0.5, dtype)
+    torch.testing.assert_close(got.float(), ref, **tol(dtype))
+    one = run_attention(k, [q[-1:]], [kx], [vx], P, dtype)
+    assert torch.equal(one[0], got[-1])
+    for far in (0, 9999, L - 1):
+        q2, k2 = q[-1:].clone() * 0.1, kx.clone() * 0.1
+        q2[:, :, 0] = 40.0
+        k2[far, :, 0] = 40.0
+        out = run_attention(k, [q2], [k2], [vx], P, dtype)
+        torch.testing.assert_close(out[0].float(), vx[far].float().repeat_interleave(nq, dim=0), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_attention_far_key_in_prompt_rows(dtype):
     """A key that outweighs all others, seen from the rows of a late portion of a prompt: every row at
     or after it must return its value, through the kernel that shares tiles and the other one.  Then
