@@ -14,17 +14,22 @@
 // any cut of a sequence into steps, and any split of the keys over waves and
 // workgroups, gives the same bits:
 //   tile     64 keys, positions 64t .. 64t+63.  Each tile is reduced on its
-//            own: m = max of the visible scores, p = 2^(s - m), l = sum p,
-//            acc = P V accumulated from zero.  A tile without a visible key is
-//            empty (m = -inf).
+//            own: m = (max of the visible raw scores) * c with c = scale * log2(e),
+//            p = 2^(fma(raw, c, -m)), l = sum p, acc = P V accumulated from zero.
+//            A tile without a visible key is empty (m = -inf).
 //   segment  4 tiles (256 keys).  Its non-empty tiles are folded, ascending,
 //            into a state that starts empty:
 //              M' = max(M, m); ACC' = fma(acc, 2^(m - M'), ACC * 2^(M - M')); L' likewise.
 //   total    the non-empty segments are folded, ascending, the same way.
-// The prompt kernel folds in registers as it walks the tiles.  The decode
-// kernel gives every tile of a segment to a wave of its own, folds the four in
-// LDS and leaves the segment's (m, l, acc) in a scratch buffer that
-// attn_combine folds; the arithmetic is the same sequence of fp32 operations.
+// Kernels, all with the same sequence of fp32 operations per row:
+//   attn_prefill_lds   prompt rows, head sizes 64/128/256 and pages of a tile or more: key and value
+//                      tiles pass through LDS once per workgroup; folds in registers.
+//   attn_prefill       prompt rows of every shape: fragments straight from global memory.
+//   attn_decode        decoded tokens: every tile of a segment has a wave of its own, the four are
+//                      folded in LDS, the segment's (m, l, acc) goes to a scratch buffer ...
+//   attn_combine       ... which this one folds.
+//   attn_decode_whole  decoded tokens of large batches: all tiles of a token and kv head in one
+//                      workgroup, folded from LDS; no scratch.
 //
 // Cache layout: keys [pages, nkv, page, d]; values transposed [pages, nkv, d, page],
 // so that both MFMA operands of both products are 16-byte loads from global
