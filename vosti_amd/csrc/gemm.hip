@@ -12,14 +12,18 @@
 // for the same reason (kernels/triton_kernels/matmul.py:33-73,
 // kernels/triton_kernels/qkv_matmul.py:24-32).
 //
-//   gemm_skinny: M <= 64.  Streams the weights once from HBM.  A workgroup of
-//                eight waves owns 16 weight rows; wave w takes the chunks w,
-//                w+8, ... and keeps a rolling window of W slabs (weights and
-//                activations) in flight, also across chunk borders.  After each
-//                round of eight chunks the chunk sums meet in LDS and are added
-//                in chunk order.
-//   gemm_tiled:  any M.  128x128 output tile per workgroup staged through LDS,
-//                64x64 per wave; a second accumulator set holds the total.
+//   gemm_stream         M <= 64, K a multiple of 512.  Streams the weights once from HBM: persistent
+//                       workgroups of eight waves walk over 16-row weight tiles (one or two at a time);
+//                       wave w takes the chunks w, w+8, ... and keeps a rolling window of slabs in
+//                       flight, also across tile borders.  After each round of eight chunks the chunk
+//                       sums meet in LDS and are added in chunk order.
+//   gemm_stream_swiglu  the same for the gate/up projection with SwiGLU folded in (M <= 16).
+//   gemm_skinny         M <= 64, any K: the same decomposition with predicated loads.
+//   gemm_pipe           any M, K a multiple of two slabs (128 bytes of a row): 128x128 output tile per
+//                       workgroup, 64x64 per wave, tiles straight from global memory into LDS, two
+//                       stages; a second accumulator set holds the total.  Optionally SwiGLU in the
+//                       epilogue.
+//   gemm_tiled          any M and K: the same tile through registers into LDS, predicated.
 #include "common.h"
 #include "mma.h"
 #include "vec.h"
