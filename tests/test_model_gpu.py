@@ -264,3 +264,41 @@ def test_layers_of_full_width(full_width_dir, dtype_name):
         got = replay(make_runner(d, dtype_name, 64, num_pages=pages), steps)
         bad = [k for k in sorted(whole) if not torch.equal(got[k], whole[k])]
         assert set(got) == set(whole) and not bad, f"{label}: first differing (request, position) {bad[:1]} of {len(bad)}"
+
+
+SWEEP = [
+    # hidden, layers, q heads, kv heads, head size, inside, vocab, page, eps, theta, tied
+    (80, 1, 3, 3, 80, 96, 211, 32, 1e-6, 1e4, True),        # one q head per kv head, head size 80
+    (128, 2, 8, 1, 64, 200, 777, 128, 1e-5, 1e6, False),    # eight q heads on one kv head, pages of two tiles
+    (512, 1, 6, 2, 128, 520, 300, 64, 1e-6, 5e5, False),    # width of one chunk, groups of three
+    (96, 2, 2, 2, 48, 64, 97, 8, 1e-5, 1e5, True),          # head size 48, the smallest page
+    (1024, 1, 2, 1, 256, 1032, 130, 64, 1e-6, 1e6, False),  # head size 256, two chunks
+]
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+@pytest.mark.parametrize("case", range(len(SWEEP)))
+def test_other_shapes(tmp_path_factory, case, dtype_name):
+    """Shapes that take other kernels or other branches of them than the tiny configurations do (head
+    sizes 48, 80 and 256, groups of 1, 3 and 8 q heads, pages of 8 to 128, widths of one and two chunks):
+    whole prompts against the plain implementation, two cuttings against the whole prompts bit for bit."""
+    from vosti_amd.config import Qwen3Config
+    from vosti_amd.weights import write_random_model
+    H, L, nq, nkv, d, I, V, page, eps, theta, tied = SWEEP[case]
+    cfg = dict(vocab_size=V, hidden_size=H, intermediate_size=I, num_hidden_layers=L, num_attention_heads=nq,
+               num_key_value_heads=nkv, head_dim=d, max_position_embeddings=320, rms_norm_eps=eps, rope_theta=theta,
+               tie_word_embeddings=tied)
+    folder = tmp_path_factory.mktemp(f"sweep_{case}")
+    write_random_model(Qwen3Config(**cfg), 30 + case, folder, dtype=torch.bfloat16)
+    rng = random.Random(50 + case)
+    prompts = [[rng.randrange(V) for _ in range(n)] for n in (3, 70, 129, 300)]
+    plain = PlainQwen3(folder, DTYPES[dtype_name])
+    pages = -(-300 // page) + 1
+    whole = replay(make_runner(folder, dtype_name, page, num_pages=pages), cut_whole(prompts))
+    for i, p in enumerate(prompts):
+        got = torch.stack([whole[(i, j)] for j in range(len(p))])
+        torch.testing.assert_close(got, plain.logits(p), **TOL[dtype_name], msg=lambda m: f"case {case}, request {i}: {m}")
+    for label, steps in (("tail", cut_tail(prompts)), ("chunks", cut_chunks(prompts))):
+        got = replay(make_runner(folder, dtype_name, page, num_pages=pages), steps)
+        bad = [k for k in sorted(whole) if not torch.equal(got[k], whole[k])]
+        assert set(got) == set(whole) and not bad, f"case {case}, {label}: first differing (request, position) {bad[:1]} of {len(bad)}"
