@@ -493,7 +493,7 @@ def test_attention_refuses_bad_sizes():
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,I,K", [(8, 100, 1024), (16, 256, 4096), (1, 33, 512), (5, 48, 96), (20, 64, 1024),
-                                   (100, 100, 1024), (300, 256, 2048), (129, 70, 192), (130, 64, 96)])
+                                   (100, 100, 1024), (300, 256, 2048), (129, 70, 192), (130, 64, 96), (40, 8200, 128)])
 def test_gemm_swiglu_fused_equals_separate(dtype, M, I, K):
     """The gate/up projection with the activation folded in (the streaming kernel for few rows, the
     pipelined tile kernel for many) gives the bits of the two separate kernels; (5, 48, 96),

@@ -712,7 +712,9 @@ int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K
 // 1: the streaming kernel (few rows), 2: the pipelined tile kernel (many rows), 0: neither.
 int vk_gemm_swiglu_supported(int M, int I, int K) {
   if (M >= 1 && M <= 16 && I > 0 && K % KC == 0 && K <= SK_WAVES * KC) return 1;
-  if (M > 64 && I > 0 && K % (2 * VK_SLAB) == 0) return 2;
+  // Where vk_gemm would take the pipelined kernel for the [2I, K] weight: more than 64 rows, or more than 32
+  // with many weight rows.
+  if ((M > 64 || (M > 32 && 2 * I >= 16384)) && I > 0 && K % (2 * VK_SLAB) == 0) return 2;
   return 0;
 }
 
