@@ -39,7 +39,10 @@ def test_gemm(dtype, M, N, K):
     got_t = k.gemm(a.cuda(), w.cuda(), kernel=2)
     torch.testing.assert_close(got_t.float().cpu(), ref.to(dtype).float(), **tol(dtype))
     if M <= 64:
-        for code in (1, 7, 0):    # one and two weight tiles per workgroup, and the kernel chosen by size
+        codes = [1, 7, 0]           # one and two weight tiles per workgroup, and the kernel chosen by size
+        if M > 16 and K % 512 == 0:
+            codes += [8, 9]         # activations shared through LDS, two and four chunks in work
+        for code in codes:
             got_s = k.gemm(a.cuda(), w.cuda(), kernel=code)
             assert torch.equal(got_s, got_t), f"the skinny kernel {code} and the tiled kernel must agree bitwise"
     # A row of a batch equals the same row alone, bitwise.

@@ -636,12 +636,174 @@ static int launch_pipe(elem_t* out, const elem_t* act, const elem_t* w, int M, i
   return vk_check_launch("gemm_pipe");
 }
 
+// ------------------------------------------------------------------ mid
+// 17 to 64 rows.  The streaming kernels read all activations once per 16 weight rows, which at 64 rows
+// is four times the weights and binds them to the second-level cache.  Here a workgroup of eight waves
+// takes 64 weight rows: wave (nt, kh) streams weight tile nt (16 rows) for the chunks kh, kh + 2, ...
+// into registers with a rolling window, as the streaming kernels do, and the activations of the two
+// chunks in work go into LDS once for all waves (global_load_lds, a quarter chunk at a time, two
+// buffers).  After a pair of chunks the waves with kh = 1 hand their chunk sum over through LDS and the
+// waves with kh = 0 add both to the total, in chunk order.  K is a multiple of 512.
+//
+// Waits: the barrier of a step is a bare s_barrier (a __syncthreads would wait for every weight load in
+// flight); a wave waits for its part of the activation loads by count: they are followed by exactly
+// MID_QS weight loads before the next step begins (MID_W at the start), kept so by scheduling barriers.
+#define MID_QS 4                       // slabs per step
+#define MID_W 8                        // weight slabs in flight per wave
+__device__ __forceinline__ void mid_wait_vmcnt_4() { __builtin_amdgcn_s_waitcnt(0x0F74); }
+__device__ __forceinline__ void mid_wait_vmcnt_w() { static_assert(MID_W == 8, "vmcnt(8)"); __builtin_amdgcn_s_waitcnt(0x0F78); }
+__device__ __forceinline__ void mid_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+__device__ __forceinline__ void mid_load_to_lds16(const elem_t* src, unsigned char* dst) {
+  __builtin_amdgcn_global_load_lds(src, (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+}
+
+template <int MT, int KH>
+__global__ __launch_bounds__(512) void gemm_mid_kernel(elem_t* __restrict__ out, const elem_t* __restrict__ act,
+                                                       const elem_t* __restrict__ w, int M, int N, int K,
+                                                       int64_t lda, int64_t ldo, int out_vec_ok) {
+  constexpr int NTW = 8 / KH;                       // weight tiles of the workgroup (16 rows each)
+  constexpr int STEPS = KC_SLABS / MID_QS;          // steps per chunk
+  constexpr int ROW_B = MID_QS * 64;                // bytes of an activation row in a step: 256
+  constexpr int HALF_B = 16 * MT * ROW_B;           // one chunk's part of a buffer
+  constexpr int BUF_B = KH * HALF_B;
+  constexpr int DMA = MT * KH / 2;                  // activation loads per wave and step (8 KH MT / 2 in all... 4 rows each)
+  static_assert((MT * KH) % 2 == 0, "the activation loads divide evenly over the waves");
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];   // [2 buffers][kh][16 MT rows][256 B], then part
+  f32x4* part = reinterpret_cast<f32x4*>(lds + 2 * BUF_B);              // [KH - 1][NTW tiles][MT][64 lanes]
+
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r16 = lane & 15, kg = lane >> 4;
+  const int nt = wave % NTW, kh = wave / NTW;
+  const int nchunks = K / KC, ngroups = (nchunks + KH - 1) / KH;     // group: KH chunks in work together
+  const int nsteps = ngroups * STEPS;
+  const int last_full = nchunks - (ngroups - 1) * KH;                // chunks of the last group: 1 .. KH
+
+  // Weights: row of this wave's tile, chunk sequence kh, kh + KH, ...; a chunk beyond the last is read as
+  // the last (and not used), so that every wave issues the same number of loads.
+  const elem_t* wrow = w + (int64_t)min((int)blockIdx.x * 16 * NTW + nt * 16 + r16, N - 1) * K + kg * VK_VEC;
+  frag_t wbuf[MID_W];
+  auto issue_w = [&](int g, int slot) {              // g: this wave's slab number; slot = g % MID_W
+    const int gg = min(g, nsteps * MID_QS - 1);
+    const int c = min(KH * (gg / KC_SLABS) + kh, nchunks - 1);
+    wbuf[slot] = *reinterpret_cast<const frag_t*>(wrow + (int64_t)c * KC + (gg % KC_SLABS) * VK_SLAB);
+  };
+  // Activations of a step: KH * 16 MT rows of 256 bytes; a wave-level load fills 4 rows, lane i the
+  // 16-byte column i % 16 of row i / 16, which holds the logical column (i % 16) ^ (row % 16).
+  const elem_t* asrc[DMA];
+  int adst[DMA], ah[DMA];
+#pragma unroll
+  for (int j = 0; j < DMA; ++j) {
+    const int id = wave * DMA + j;                   // 0 .. 4 MT KH - 1
+    const int h = id / (4 * MT), row = (id % (4 * MT)) * 4 + (lane >> 4);
+    ah[j] = h;
+    asrc[j] = act + (int64_t)min(row, M - 1) * lda + (((lane & 15) ^ (row & 15)) * VK_VEC);
+    adst[j] = h * HALF_B + (id % (4 * MT)) * 4 * ROW_B;
+  }
+  auto issue_a = [&](int t) {                        // step t of the workgroup
+    const int tt = min(t, nsteps - 1);
+    const int group = tt / STEPS, q = tt % STEPS;
+    unsigned char* base = lds + (t & 1) * BUF_B;
+#pragma unroll
+    for (int j = 0; j < DMA; ++j) {
+      const int c = min(group * KH + ah[j], nchunks - 1);    // beyond the last chunk: the last again (not used)
+      mid_load_to_lds16(asrc[j] + (int64_t)c * KC + q * MID_QS * VK_SLAB, base + adst[j]);
+    }
+  };
+
+  f32x4 acc[MT], total[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc[mt] = total[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // The chunk sums of a complete group join the total in chunk order: this wave's own, then the others'.
+  auto close_group = [&](int chunks_in_group) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      total[mt].x = total[mt].x + acc[mt].x; total[mt].y = total[mt].y + acc[mt].y;
+      total[mt].z = total[mt].z + acc[mt].z; total[mt].w = total[mt].w + acc[mt].w;
+#pragma unroll
+      for (int h = 1; h < KH; ++h) {
+        if (h < chunks_in_group) {
+          const f32x4 p = part[(((h - 1) * NTW + nt) * MT + mt) * 64 + lane];
+          total[mt].x = total[mt].x + p.x; total[mt].y = total[mt].y + p.y;
+          total[mt].z = total[mt].z + p.z; total[mt].w = total[mt].w + p.w;
+        }
+      }
+    }
+  };
+
+  issue_a(0);
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int i = 0; i < MID_W; ++i) issue_w(i, i);
+  __builtin_amdgcn_sched_barrier(0);
+  constexpr int TURN = MID_W / MID_QS;      // steps in one turn of the weight window
+  static_assert(STEPS % TURN == 0, "a turn of the weight window is a whole number of steps");
+  for (int t2 = 0; t2 < nsteps; t2 += TURN) {
+#pragma unroll
+   for (int u = 0; u < TURN; ++u) {         // written out: the window's slots are then fixed registers
+    const int t = t2 + u;
+    if (t == 0) mid_wait_vmcnt_w(); else mid_wait_vmcnt_4();
+    mid_barrier();          // step t's activations are in LDS; everyone is done with the other buffer
+    const int group = t / STEPS, q = t % STEPS;
+    if (q == 0 && group > 0) {
+      if (kh == 0) close_group(KH);           // the group before is complete
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    issue_a(t + 1);
+    __builtin_amdgcn_sched_barrier(0);
+    const unsigned char* abase = lds + (t & 1) * BUF_B + kh * HALF_B;
+#pragma unroll
+    for (int s = 0; s < MID_QS; ++s) {
+      const int g = t * MID_QS + s;
+      const frag_t fw = wbuf[u * MID_QS + s];
+      frag_t fa[MT];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+        fa[mt] = *reinterpret_cast<const frag_t*>(abase + (mt * 16 + r16) * ROW_B + (((s * 4 + kg) ^ r16) << 4));
+      issue_w(g + MID_W, u * MID_QS + s);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) acc[mt] = mma_slab(fw, fa[mt], acc[mt]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (q == STEPS - 1 && kh > 0) {
+      // This wave's chunk of the group is complete: hand it over (one beyond the last chunk is not used).
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) part[(((kh - 1) * NTW + nt) * MT + mt) * 64 + lane] = acc[mt];
+    }
+   }
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);      // the loads issued beyond the end
+  mid_barrier();
+  if (kh == 0) {
+    close_group(last_full);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+      store_out4(out, ldo, mt * 16 + r16, blockIdx.x * 16 * NTW + nt * 16 + 4 * kg, M, N, total[mt], out_vec_ok);
+  }
+}
+
+template <int MT, int KH>
+static int launch_mid(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K, int64_t lda, int64_t ldo,
+                      int vec_ok, hipStream_t st) {
+  constexpr int NTW = 8 / KH;
+  const size_t smem = (size_t)2 * KH * 16 * MT * (MID_QS * 64) + (size_t)(KH - 1) * NTW * MT * 64 * sizeof(f32x4);
+  static bool configured = false;
+  if (!configured) {
+    (void)hipFuncSetAttribute((const void*)gemm_mid_kernel<MT, KH>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    configured = true;
+  }
+  gemm_mid_kernel<MT, KH><<<(N + 16 * NTW - 1) / (16 * NTW), 512, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok);
+  return vk_check_launch("gemm_mid");
+}
+
 // ==================================================================== host
 extern "C" {
 
 // kernel: 0 = choose by size, 1 = skinny (M <= 64), 2 = tiled (pipelined if K allows), 3 = tiled through
 // registers, 4..6 = pipelined with 2..4 stages, 7 = skinny with two weight tiles per workgroup where it has
-// such a variant (for measurements and tests).  The result does not depend on the choice.
+// such a variant, 8 and 9 = activations shared through LDS with 64 and 32 weight rows per workgroup (17 to
+// 64 rows; for measurements and tests).  The result does not depend on the choice.
 int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K, int64_t lda, int64_t ldo,
             int kernel, hipStream_t st) {
   VK_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
@@ -650,17 +812,32 @@ int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K
              (long long)lda, VK_VEC);
   VK_REQUIRE(ldo >= N, "gemm: output row stride %lld is smaller than N=%d", (long long)ldo, N);
   VK_REQUIRE(((uintptr_t)act % 16) == 0 && ((uintptr_t)w % 16) == 0, "gemm: operands must be 16-byte aligned");
-  VK_REQUIRE(kernel >= 0 && kernel <= 7, "gemm: unknown kernel %d", kernel);
+  VK_REQUIRE(kernel >= 0 && kernel <= 9, "gemm: unknown kernel %d", kernel);
   if (M == 0) return 0;
   const int vec_ok = (ldo % 4 == 0) && ((uintptr_t)out % 16 == 0);
-  // Measured on Qwen3-8B shapes (MI355X).  Up to 16 rows: the streaming kernel.  17 to 64 rows: the
-  // streaming kernel with two weight tiles per workgroup where that still leaves some 200 workgroups
-  // (6144 weight rows), with one tile below that, and the pipelined tile kernel for many weight rows
-  // and more than 32 rows.  More rows: the pipelined tile kernel.
+  // Measured on Qwen3-8B shapes (MI355X).  Up to 16 rows: the streaming kernel.  17 to 64 rows with K in
+  // whole chunks: with 16384 weight rows or more the kernel that shares activations through LDS, 64
+  // weight rows per workgroup; with fewer, its variant with 32 weight rows from 41 rows on, and below
+  // that the streaming kernel, with two weight tiles per workgroup from 6144 weight rows on.  More
+  // rows: the pipelined tile kernel.
   if (kernel == 0) {
     if (M <= 16) kernel = 1;
+    else if (M <= 64 && K % KC == 0) kernel = N >= 16384 ? 8 : (M > 40 ? 9 : (N >= 6144 ? 7 : 1));
     else if (M <= 64) kernel = (N >= 16384 && M > 32) ? 2 : (N >= 6144 ? 7 : 1);
     else kernel = 2;
+  }
+  if (kernel == 8 || kernel == 9) {
+    VK_REQUIRE(M > 16 && M <= 64 && K % KC == 0, "gemm: the mid kernel takes 17 to 64 rows and K a multiple of %d", KC);
+    const int mt = (M + 15) / 16;
+    if (kernel == 8) {      // 64 weight rows per workgroup, two chunks in work
+      if (mt == 2) return launch_mid<2, 2>(out, act, w, M, N, K, lda, ldo, vec_ok, st);
+      if (mt == 3) return launch_mid<3, 2>(out, act, w, M, N, K, lda, ldo, vec_ok, st);
+      return launch_mid<4, 2>(out, act, w, M, N, K, lda, ldo, vec_ok, st);
+    }
+    // 32 weight rows per workgroup, four chunks in work
+    if (mt == 2) return launch_mid<2, 4>(out, act, w, M, N, K, lda, ldo, vec_ok, st);
+    if (mt == 3) return launch_mid<3, 4>(out, act, w, M, N, K, lda, ldo, vec_ok, st);
+    return launch_mid<4, 4>(out, act, w, M, N, K, lda, ldo, vec_ok, st);
   }
   if (kernel == 1 || kernel == 7) {
     VK_REQUIRE(M <= 64, "gemm: the skinny kernel takes at most 64 rows, got %d", M);
@@ -712,9 +889,7 @@ int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K
 // 1: the streaming kernel (few rows), 2: the pipelined tile kernel (many rows), 0: neither.
 int vk_gemm_swiglu_supported(int M, int I, int K) {
   if (M >= 1 && M <= 16 && I > 0 && K % KC == 0 && K <= SK_WAVES * KC) return 1;
-  // Where vk_gemm would take the pipelined kernel for the [2I, K] weight: more than 64 rows, or more than 32
-  // with many weight rows.
-  if ((M > 64 || (M > 32 && 2 * I >= 16384)) && I > 0 && K % (2 * VK_SLAB) == 0) return 2;
+  if (M > 64 && I > 0 && K % (2 * VK_SLAB) == 0) return 2;
   return 0;
 }
 
