@@ -18,6 +18,8 @@
 //                       flight, also across tile borders.  After each round of eight chunks the chunk
 //                       sums meet in LDS and are added in chunk order.
 //   gemm_stream_swiglu  the same for the gate/up projection with SwiGLU folded in (M <= 16).
+//   gemm_mid            17 <= M <= 64, K a multiple of 512: 64 or 32 weight rows per workgroup, weights
+//                       streamed into registers, the activations of the chunks in work shared through LDS.
 //   gemm_skinny         M <= 64, any K: the same decomposition with predicated loads.
 //   gemm_pipe           any M, K a multiple of two slabs (128 bytes of a row): 128x128 output tile per
 //                       workgroup, 64x64 per wave, tiles straight from global memory into LDS, two
