@@ -2,6 +2,8 @@
 """Decode and prefill throughput of the Qwen3-8B shape with random weights on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L]
+    python bench.py --workload mixed14b     # Qwen3-14B shape: 32 prompts of 128 to 4,096 tokens, prefill in portions beside decoding
+    python bench.py --workload prefix32b    # Qwen3-32B shape: 64 requests at context 8,192 that share a 1,024-token prefix
 
 A step is one decode step of the engine (plan, forward, sample, commit) for a
 batch of B requests whose prompts of 2,048 random tokens were prefilled through
@@ -25,6 +27,9 @@ sys.path.insert(0, str(Path(__file__).resolve().parent))
 QWEN3_8B = dict(vocab_size=151936, hidden_size=4096, intermediate_size=12288, num_hidden_layers=36,
                 num_attention_heads=32, num_key_value_heads=8, head_dim=128, max_position_embeddings=40960,
                 rms_norm_eps=1e-6, rope_theta=1e6, tie_word_embeddings=False)
+# The two larger shapes of the same family, for the other workloads.
+QWEN3_14B = dict(QWEN3_8B, hidden_size=5120, intermediate_size=17408, num_hidden_layers=40, num_attention_heads=40)
+QWEN3_32B = dict(QWEN3_8B, hidden_size=5120, intermediate_size=25600, num_hidden_layers=64, num_attention_heads=64)
 PROMPT_TOKENS = 2048
 GENERATED_TOKENS = 256
 HBM_PEAK_GBS = 8000.0
@@ -55,11 +60,12 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=None, help="requests (default 8; 64 for prefix32b)")
     ap.add_argument("--layers", type=int, default=QWEN3_8B["num_hidden_layers"])
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--graphs", type=int, default=1, choices=[0, 1], help="replay decode steps from captured HIP graphs")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill timing")
+    ap.add_argument("--workload", default="decode8b", choices=["decode8b", "mixed14b", "prefix32b"])
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -75,6 +81,10 @@ def main() -> int:
     from vosti_amd.sampling import SamplingParams
     from vosti_amd.weights import random_weights_on_gpu
 
+    if args.workload != "decode8b":
+        return other_workload(args)
+    if args.batch is None:
+        args.batch = 8
     cfg = Qwen3Config(**dict(QWEN3_8B, num_hidden_layers=args.layers))
     model = build_model(cfg, args.dtype)
     random_weights_on_gpu(model, seed=0)
@@ -152,6 +162,125 @@ def main() -> int:
             s, _ = decode_run(B, min(args.steps, 32), min(args.warmup, 4))
             points[name] = round(B / s, 2)
         record["points"] = points
+    print(json.dumps(record), flush=True)
+    return 0
+
+
+def progress(text: str, state={"t": 0.0}) -> None:
+    """A line on stderr, at most every ten seconds: long runs show that they are alive."""
+    now = time.perf_counter()
+    if now - state["t"] >= 10.0:
+        state["t"] = now
+        print(f"bench.py: {text}", file=sys.stderr, flush=True)
+
+
+def other_workload(args) -> int:
+    """The two larger shapes with the workloads named for them: one JSON line each, same fields."""
+    import torch
+    from vosti_amd.config import Qwen3Config
+    from vosti_amd.engine import Engine
+    from vosti_amd.models import build_model
+    from vosti_amd.sampling import SamplingParams
+    from vosti_amd.weights import random_weights_on_gpu
+
+    shape = QWEN3_14B if args.workload == "mixed14b" else QWEN3_32B
+    full_layers = shape["num_hidden_layers"]
+    layers = args.layers if args.layers != QWEN3_8B["num_hidden_layers"] else full_layers
+    cfg = Qwen3Config(**dict(shape, num_hidden_layers=layers))
+    print(f"bench.py: {args.workload}: building {layers} layers", file=sys.stderr, flush=True)
+    model = build_model(cfg, args.dtype)
+    random_weights_on_gpu(model, seed=0)
+    torch.cuda.synchronize()
+    print("bench.py: weights ready", file=sys.stderr, flush=True)
+    elem = 2 if args.dtype == "bfloat16" else 4
+    dt_name = "bf16" if args.dtype == "bfloat16" else "fp32"
+    rng = random.Random(1)
+    page = 64
+    name = "Qwen3-14B shape" if args.workload == "mixed14b" else "Qwen3-32B shape"
+    base = {"n_gpus": 1, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dt_name,
+            "data": "synthetic: seeded random token prompts, seeded random weights", "unit": "tokens/s"}
+    shape_keys = {"model": name, "layers": layers, "layers_of_model": full_layers, "hidden_size": cfg.hidden_size,
+                  "intermediate_size": cfg.intermediate_size, "q_heads": cfg.num_attention_heads,
+                  "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim, "vocab_size": cfg.vocab_size,
+                  "page_size": page, "parallelism": "single GPU", "graphs": bool(args.graphs)}
+
+    if args.workload == "mixed14b":
+        # 32 prompts of 128 to 4,096 tokens, 128 new tokens each; prompts enter in portions of at most 4,096
+        # tokens a step beside the decoding of the requests that are further on.
+        n, new = 32, 128
+        lengths = [rng.randint(128, 4096) for _ in range(n)]
+        prompts = [[rng.randrange(cfg.vocab_size) for _ in range(L)] for L in lengths]
+        pages = sum(-(-(L + new + 1) // page) for L in lengths) + 8
+        eng = Engine(model, num_pages=pages, page_size=page, max_num_seqs=n, max_num_batched_tokens=4096,
+                     enable_prefix_cache=False, graphs=bool(args.graphs))
+        sp = SamplingParams(max_tokens=new, ignore_eos=True)
+        for p_ in prompts:
+            eng.add_request(p_, sp)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        steps = emitted = 0
+        while eng.has_unfinished():
+            emitted += len(eng.step())
+            steps += 1
+            progress(f"step {steps}, {emitted} tokens out")
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        assert emitted == n * new
+        layers_w, head_w = gemm_params(cfg)
+        flops = 2.0 * (sum(lengths) + n * new) * layers_w + 2.0 * n * new * head_w
+        record = dict(base, metric="tokens/s through a mixed batch: 32 prompts of 128-4,096 tokens in portions beside decoding, Qwen3-14B shape",
+                      value=round((sum(lengths) + emitted) / dt, 1), steps=steps, warmup=0, ms_per_step=round(dt / steps * 1e3, 3),
+                      config=dict(shape_keys, global_batch=n, prompt_tokens=sum(lengths), new_tokens=emitted, token_budget=4096),
+                      output={"value": round(emitted / dt, 1), "wall_s": round(dt, 3)},
+                      roofline={"bound": "mfma", "achieved": round(flops / dt / 1e12, 1), "peak": PEAK_FLOPS[dt_name] / 1e12,
+                                "unit": "TFLOP/s (projections only)", "frac": round(flops / dt / PEAK_FLOPS[dt_name], 4)})
+        print(json.dumps(record), flush=True)
+        return 0
+
+    # prefix32b: 64 requests whose prompts share their first 1,024 tokens and go on with 7,168 of their own;
+    # the pages of the shared part are computed once and reused.  Decode steps are timed at context ~8,200.
+    n, shared_len, own_len = args.batch or 64, 1024, 7168
+    shared = [rng.randrange(cfg.vocab_size) for _ in range(shared_len)]
+    prompts = [shared + [rng.randrange(cfg.vocab_size) for _ in range(own_len)] for _ in range(n)]
+    # The first requests decode while the later ones are still prefilled, one a step: room for that too.
+    total = args.steps + args.warmup + n + 16
+    pages = shared_len // page + n * (-(-(own_len + total + 1) // page)) + 8
+    eng = Engine(model, num_pages=pages, page_size=page, max_num_seqs=n, max_num_batched_tokens=8192,
+                 enable_prefix_cache=True, graphs=bool(args.graphs))
+    sp = SamplingParams(max_tokens=total, ignore_eos=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    # The first request alone, so that its pages are published before the others look for them.
+    eng.add_request(prompts[0], sp)
+    eng.step()
+    for p_ in prompts[1:]:
+        eng.add_request(p_, sp)
+    while eng.scheduler.num_waiting() or any(eng.cache.length(r) < shared_len + own_len for r in range(n)):
+        eng.step()
+        progress(f"prefill: {eng.scheduler.num_waiting()} requests waiting")
+    torch.cuda.synchronize()
+    prefill_s = time.perf_counter() - t0
+    print(f"bench.py: prefill done in {prefill_s:.1f} s", file=sys.stderr, flush=True)
+    for _ in range(args.warmup):
+        assert len(eng.step()) == n
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        eng.step()
+    torch.cuda.synchronize()
+    step_s = (time.perf_counter() - t0) / args.steps
+    ctx = sum(eng.cache.length(r) for r in range(n)) / n - (args.steps - 1) / 2.0     # mean keys a request reads in a timed step
+    layers_w, head_w = gemm_params(cfg)
+    kv_token = 2 * cfg.num_key_value_heads * cfg.head_dim * cfg.num_hidden_layers
+    unique = (layers_w + head_w + (n * (ctx - shared_len) + shared_len) * kv_token) * elem     # shared pages once
+    record = dict(base, metric=f"decode tok/s at batch {n}, context 8,192, a 1,024-token prefix shared through the page cache, Qwen3-32B shape",
+                  value=round(n / step_s, 1), steps=args.steps, warmup=args.warmup, ms_per_step=round(step_s * 1e3, 3),
+                  config=dict(shape_keys, global_batch=n, seq_len=shared_len + own_len + total, shared_prefix=shared_len,
+                              context_at_timing=round(ctx), reused_prefix_pages=eng.cache.prefix_hits()),
+                  prefill={"value": round((n * own_len + shared_len) / prefill_s, 1), "tokens": n * own_len + shared_len,
+                           "ms": round(prefill_s * 1e3, 1)},
+                  roofline={"bound": "hbm", "achieved": round(unique / step_s / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                            "frac": round(unique / step_s / 1e9 / HBM_PEAK_GBS, 4)})
     print(json.dumps(record), flush=True)
     return 0
 

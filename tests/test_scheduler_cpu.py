@@ -220,6 +220,28 @@ def test_prefix_reuse_through_the_scheduler():
     assert cache.prefix_hits() == 3
 
 
+def test_reuse_is_counted_once_for_an_admission_that_had_to_wait():
+    """A request whose prompt finds cached pages but no pages for the rest waits; each step tries its
+    admission again, and only the one that stands counts as a reuse."""
+    cache, s = make(page=4, pages=7, prefix=True)
+    shared = list(range(50, 58))                                   # two pages
+    h = {0: shared + list(range(8)), 1: shared + list(range(20, 32))}
+    s.add_request(0, h[0], 6)                                      # 4 pages for its prompt, 2 more while decoding
+    s.plan(); s.commit([toy_next(h[0])]); h[0].append(toy_next(h[0][:16]))
+    s.add_request(1, h[1], 2)                                      # 3 pages of its own and one to decode into: 7 - 4 do not hold them
+    waited = 0
+    while s.num_waiting():
+        rows = s.plan()
+        assert cache.check() == ""
+        waited += 1
+        s.commit([toy_next(h[r.request_id]) for r in rows if r.sample])
+        for r in rows:
+            if r.sample:
+                h[r.request_id].append(toy_next(h[r.request_id]))
+    assert waited > 2
+    assert cache.prefix_hits() == 2 and cache.prefix_hit_requests() == 1
+
+
 @pytest.mark.parametrize("seed", range(6))
 def test_outputs_do_not_depend_on_the_schedule(seed):
     """Staggered arrivals, small budgets, few pages, windows: every request still gets the tokens it

@@ -142,6 +142,7 @@ Status CacheManager::add_request(RequestId id, const int32_t* prompt, int n_prom
     }
     r.length = r.published * page_size_;
     r.tokens.assign(prompt, prompt + r.length);
+    r.attached = r.published;
     prefix_hit_pages_ += r.published;
     if (r.published > 0) ++prefix_hit_requests_;
     if (cached_tokens) *cached_tokens = r.length;
@@ -166,6 +167,7 @@ Status CacheManager::extend(RequestId id, const int32_t* tokens, int n) {
   const Status st = grow(r, r.length + n, /*all_keys_only=*/false);
   if (st != OK) return st;
   r.tokens.insert(r.tokens.end(), tokens, tokens + n);
+  r.ran = true;
   r.pending = n;
   return OK;
 }
@@ -246,6 +248,10 @@ Status CacheManager::finish(RequestId id) {
   auto it = requests_.find(id);
   if (it == requests_.end()) return UNKNOWN_REQUEST;
   Request& r = it->second;
+  if (!r.ran && r.attached > 0) {
+    prefix_hit_pages_ -= r.attached;
+    prefix_hit_requests_ -= 1;
+  }
   const int n_logical = r.pages.empty() ? 0 : (int)r.pages[0].size();
   // Tail to root, so that in the cached queue children stand before parents.
   for (int j = n_logical - 1; j >= 0; --j) {

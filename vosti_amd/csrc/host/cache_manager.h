@@ -86,7 +86,9 @@ class CacheManager {
   Status fill_block_table(RequestId id, int group, int32_t* out, int width) const;
   Status fill_slots(RequestId id, int group, int start, int n, int32_t* out) const;
 
-  // Counters for tests and logs.
+  // Counters for tests and logs.  An admission that is taken back before any
+  // step was planned for the request (no pages for the rest of its prompt)
+  // leaves them as they were.
   int64_t prefix_hits() const { return prefix_hit_pages_; }
   int64_t prefix_hit_requests() const { return prefix_hit_requests_; }   // admissions that found a cached prefix
   int64_t evictions() const { return evictions_; }
@@ -126,6 +128,8 @@ class CacheManager {
     std::vector<int> nodes;                   // [logical page] node index or -1 (prefix cache only)
     int published = 0;                        // leading pages that are nodes of this request's chain
     bool chain_broken = false;                // a page lost the race for its hash: nothing later is published
+    int attached = 0;                         // cached pages found at admission
+    bool ran = false;                         // a step was planned for it: its admission stands in the counters
   };
 
   int take_page(int g);
