@@ -370,14 +370,41 @@ def test_attention_many_decoded_tokens(dtype):
             got = run_attention(k, q_list, kk, vv, P, dtype, window=window, poison=float("nan"))
             k.lib.vk_attn_set_decode_variant(1)
             whole = run_attention(k, q_list, kk, vv, P, dtype, window=window, poison=float("nan"), seed=4)
+            k.lib.vk_attn_set_decode_variant(3)
+            by_wave = run_attention(k, q_list, kk, vv, P, dtype, window=window, poison=float("nan"), seed=5)
         finally:
             k.lib.vk_attn_set_decode_variant(0)
-        assert torch.equal(whole, got)
+        assert torch.equal(whole, got) and torch.equal(by_wave, got)
         for i in (0, 11, 23):
             ref = plain.attention(q_list[i], kk[i], vv[i], d ** -0.5, dtype, window=window)
             torch.testing.assert_close(got[i:i + 1].float(), ref, **tol(dtype))
             alone = run_attention(k, q_list[i:i + 1], kk[i:i + 1], vv[i:i + 1], P, dtype, window=window)
             assert torch.equal(alone[0], got[i])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,d,P,window", [(16, 2, 128, 64, 0), (8, 1, 128, 128, 700), (3, 1, 64, 64, 0), (40, 2, 256, 64, 0),
+                                               (4, 2, 80, 64, 130)])
+def test_attention_decode_kernels_agree(dtype, nq, nkv, d, P, window):
+    """Decoded tokens after contexts that end at every place of a tile, a segment and a page, through
+    the kernel with a wave per tile and the one with a wave per segment (head sizes and pages it knows
+    at compile time, and one it does not): the same bits, and the plain result."""
+    k = kern(dtype)
+    lens = [1, 2, 63, 64, 65, 255, 256, 257, 320, 511, 512, 513, 1023, 1024, 1025, 1300, 1793, 2047, 2048, 2049]
+    q_list = [rand((1, nq, d), dtype, 10 + i) for i in range(len(lens))]
+    kk = [rand((n, nkv, d), dtype, 40 + i) for i, n in enumerate(lens)]
+    vv = [rand((n, nkv, d), dtype, 70 + i) for i, n in enumerate(lens)]
+    try:
+        k.lib.vk_attn_set_decode_variant(2)
+        got = run_attention(k, q_list, kk, vv, P, dtype, window=window, poison=float("nan"))
+        k.lib.vk_attn_set_decode_variant(3)
+        by_wave = run_attention(k, q_list, kk, vv, P, dtype, window=window, poison=float("nan"), seed=5)
+    finally:
+        k.lib.vk_attn_set_decode_variant(0)
+    assert torch.equal(by_wave, got)
+    for i in range(len(lens)):
+        ref = plain.attention(q_list[i], kk[i], vv[i], d ** -0.5, dtype, window=window)
+        torch.testing.assert_close(by_wave[i:i + 1].float(), ref, **tol(dtype))
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
