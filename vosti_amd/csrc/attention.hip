@@ -438,8 +438,10 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_lds_kernel(AttnArgs a
   const int n_blocks = n_items * BPI;
   int rank, head;            // rank: 0 for the last rows of the last item
   if (n_blocks % 8 == 0) {
-    const int j = lin >> 3;
-    rank = (j / a.nq) * 8 + (lin & 7);
+    // Rounds of eight ranks; every other round is dealt backwards, so that a part's long and
+    // short workgroups add up alike (with two rounds: ranks x and 15 - x on part x).
+    const int j = lin >> 3, round = j / a.nq, x = lin & 7;
+    rank = round * 8 + ((round & 1) ? 7 - x : x);
     head = j % a.nq;
   } else {
     rank = lin / a.nq;
