@@ -804,8 +804,8 @@ extern "C" {
 
 // kernel: 0 = choose by size, 1 = skinny (M <= 64), 2 = tiled (pipelined if K allows), 3 = tiled through
 // registers, 4..6 = pipelined with 2..4 stages, 7 = skinny with two weight tiles per workgroup where it has
-// such a variant, 8 and 9 = activations shared through LDS with 64 and 32 weight rows per workgroup (17 to
-// 64 rows; for measurements and tests).  The result does not depend on the choice.
+// such a variant, 8, 9 and 10 = activations shared through LDS with 64, 32 and 128 weight rows per workgroup
+// (17 to 64 rows; for measurements and tests).  The result does not depend on the choice.
 int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K, int64_t lda, int64_t ldo,
             int kernel, hipStream_t st) {
   VK_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
@@ -814,23 +814,28 @@ int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K
              (long long)lda, VK_VEC);
   VK_REQUIRE(ldo >= N, "gemm: output row stride %lld is smaller than N=%d", (long long)ldo, N);
   VK_REQUIRE(((uintptr_t)act % 16) == 0 && ((uintptr_t)w % 16) == 0, "gemm: operands must be 16-byte aligned");
-  VK_REQUIRE(kernel >= 0 && kernel <= 9, "gemm: unknown kernel %d", kernel);
+  VK_REQUIRE(kernel >= 0 && kernel <= 10, "gemm: unknown kernel %d", kernel);
   if (M == 0) return 0;
   const int vec_ok = (ldo % 4 == 0) && ((uintptr_t)out % 16 == 0);
   // Measured on Qwen3-8B shapes (MI355X).  Up to 16 rows: the streaming kernel.  17 to 64 rows with K in
-  // whole chunks: with 16384 weight rows or more the kernel that shares activations through LDS, 64
-  // weight rows per workgroup; with fewer, its variant with 32 weight rows from 41 rows on, and below
+  // whole chunks: the kernel that shares activations through LDS: 128 weight rows per workgroup from
+  // 24576 weight rows on (the activations that every workgroup reads are then half the weight bytes:
+  // 64 rows, 51200 x 5120: 158 -> 127 us), 64 from 16384 on; with fewer, 32 weight rows from 41 rows on, and below
   // that the streaming kernel, with two weight tiles per workgroup from 6144 weight rows on.  More
   // rows: the pipelined tile kernel.
   if (kernel == 0) {
     if (M <= 16) kernel = 1;
-    else if (M <= 64 && K % KC == 0) kernel = N >= 16384 ? 8 : (M > 40 ? 9 : (N >= 6144 ? 7 : 1));
+    else if (M <= 64 && K % KC == 0) kernel = N >= 24576 ? 10 : (N >= 16384 ? 8 : (M > 40 ? 9 : (N >= 6144 ? 7 : 1)));
     else if (M <= 64) kernel = (N >= 16384 && M > 32) ? 2 : (N >= 6144 ? 7 : 1);
     else kernel = 2;
   }
-  if (kernel == 8 || kernel == 9) {
+  if (kernel >= 8 && kernel <= 10) {
     VK_REQUIRE(M > 16 && M <= 64 && K % KC == 0, "gemm: the mid kernel takes 17 to 64 rows and K a multiple of %d", KC);
     const int mt = (M + 15) / 16;
+    if (kernel == 10) {     // 128 weight rows per workgroup, every wave all chunks of its tile
+      if (mt == 2) return launch_mid<2, 1>(out, act, w, M, N, K, lda, ldo, vec_ok, st);
+      return launch_mid<4, 1>(out, act, w, M, N, K, lda, ldo, vec_ok, st);
+    }
     if (kernel == 8) {      // 64 weight rows per workgroup, two chunks in work
       if (mt == 2) return launch_mid<2, 2>(out, act, w, M, N, K, lda, ldo, vec_ok, st);
       if (mt == 3) return launch_mid<3, 2>(out, act, w, M, N, K, lda, ldo, vec_ok, st);
