@@ -65,6 +65,8 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--graphs", type=int, default=1, choices=[0, 1], help="replay decode steps from captured HIP graphs")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill timing")
+    ap.add_argument("--prompt-tokens", type=int, default=PROMPT_TOKENS,
+                    help="context length of the decode measurement (the prefill figure is always of 2,048 tokens)")
     ap.add_argument("--workload", default="decode8b", choices=["decode8b", "mixed14b", "prefix32b"])
     args = ap.parse_args()
     if args.gpus != 1:
@@ -93,10 +95,11 @@ def main() -> int:
     dt_name = "bf16" if args.dtype == "bfloat16" else "fp32"
     rng = random.Random(0)
     page = 64
-    pages_per_request = -(-(PROMPT_TOKENS + GENERATED_TOKENS + 1) // page)
+    prompt_tokens = args.prompt_tokens
+    pages_per_request = -(-(max(prompt_tokens, PROMPT_TOKENS) + GENERATED_TOKENS + 1) // page)
 
-    def prompt():
-        return [rng.randrange(cfg.vocab_size) for _ in range(PROMPT_TOKENS)]
+    def prompt(n=None):
+        return [rng.randrange(cfg.vocab_size) for _ in range(prompt_tokens if n is None else n)]
 
     def decode_run(B: int, steps: int, warmup: int):
         eng = Engine(model, num_pages=B * pages_per_request, page_size=page, max_num_seqs=B, max_num_batched_tokens=4096,
@@ -104,7 +107,7 @@ def main() -> int:
         sp = SamplingParams(max_tokens=GENERATED_TOKENS, ignore_eos=True)
         for _ in range(B):
             eng.add_request(prompt(), sp)
-        while eng.scheduler.num_waiting() or any(eng.cache.length(r) < PROMPT_TOKENS for r in range(eng._next_id - B, eng._next_id)):
+        while eng.scheduler.num_waiting() or any(eng.cache.length(r) < prompt_tokens for r in range(eng._next_id - B, eng._next_id)):
             eng.step()                                   # prefill, two prompts a step
         for _ in range(warmup):
             assert len(eng.step()) == B
@@ -114,7 +117,7 @@ def main() -> int:
             eng.step()
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
-        ctx = PROMPT_TOKENS + warmup + 1 + (steps - 1) / 2.0          # mean keys per request over the timed steps
+        ctx = prompt_tokens + warmup + 1 + (steps - 1) / 2.0          # mean keys per request over the timed steps
         del eng
         torch.cuda.empty_cache()
         return dt / steps, ctx
@@ -124,7 +127,7 @@ def main() -> int:
         for i in range(reps + 1):
             eng = Engine(model, num_pages=pages_per_request, page_size=page, max_num_seqs=1, max_num_batched_tokens=PROMPT_TOKENS,
                          enable_prefix_cache=False)
-            eng.add_request(prompt(), SamplingParams(max_tokens=1))
+            eng.add_request(prompt(PROMPT_TOKENS), SamplingParams(max_tokens=1))
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             out = eng.step()
@@ -146,8 +149,8 @@ def main() -> int:
         "config": {"model": "Qwen3-8B shape", "layers": args.layers, "layers_of_model": QWEN3_8B["num_hidden_layers"],
                    "hidden_size": cfg.hidden_size, "intermediate_size": cfg.intermediate_size,
                    "q_heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
-                   "vocab_size": cfg.vocab_size, "global_batch": args.batch, "seq_len": PROMPT_TOKENS + GENERATED_TOKENS,
-                   "prompt_tokens": PROMPT_TOKENS, "context_at_timing": round(ctx), "page_size": page,
+                   "vocab_size": cfg.vocab_size, "global_batch": args.batch, "seq_len": prompt_tokens + GENERATED_TOKENS,
+                   "prompt_tokens": prompt_tokens, "context_at_timing": round(ctx), "page_size": page,
                    "parallelism": "single GPU", "graphs": bool(args.graphs)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
