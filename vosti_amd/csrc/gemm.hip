@@ -150,7 +150,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_stream_kernel(elem_t* __re
   // activations once, M * K elements beside its 16 * NT * K weights: more weight rows per workgroup
   // keep that traffic, which comes from the second-level cache, in proportion.
   static_assert(KC_SLABS % W == 0, "the window must divide a chunk");
-  static_assert(!RES || MT == 1, "resident activations are for one activation tile");
+  static_assert(!RES || MT <= 2, "resident activations are for one or two activation tiles");
   static_assert(NT * MT <= SK_WAVES, "one wave adds up each output tile");
   __shared__ f32x4 part[2][SK_WAVES][NT * MT][64];
 
@@ -167,7 +167,9 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_stream_kernel(elem_t* __re
   if (RES) {
     if (wave < nchunks) {
 #pragma unroll
-      for (int s = 0; s < KC_SLABS; ++s) abuf[s][0] = *reinterpret_cast<const frag_t*>(arow[0] + wave * KC + s * VK_SLAB);
+      for (int s = 0; s < KC_SLABS; ++s)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) abuf[s][mt] = *reinterpret_cast<const frag_t*>(arow[mt] + wave * KC + s * VK_SLAB);
     }
   }
   auto issue = [&](int tile, int c, int s, int slot) {
@@ -246,25 +248,29 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_stream_kernel(elem_t* __re
 // two projections rounded to the element type first, which is what the separate
 // GEMM and SwiGLU kernels compute (kernels/triton_kernels/silu_mul.py:64-87).
 // M <= 16, K <= 4096 (activations resident in registers).
-template <int W>
+template <int W, int MT>
 __global__ __launch_bounds__(64 * SK_WAVES) void gemm_stream_swiglu_kernel(elem_t* __restrict__ out,
                                                                            const elem_t* __restrict__ act,
                                                                            const elem_t* __restrict__ w, int M, int I,
                                                                            int K, int64_t lda, int64_t ldo,
                                                                            int out_vec_ok) {
   static_assert(KC_SLABS % W == 0, "the window must divide a chunk");
-  __shared__ f32x4 part[2][SK_WAVES][2][64];
+  static_assert(MT <= 2, "one or two activation tiles stay in registers");
+  __shared__ f32x4 part[2][SK_WAVES][2 * MT][64];
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r16 = lane & 15, kg = lane >> 4;
   const int nchunks = K / KC;
   const int ntiles = (I + 15) / 16;
-  const elem_t* arow = act + (int64_t)min(r16, M - 1) * lda + kg * VK_VEC;
 
-  frag_t wg[W], wu[W], abuf[KC_SLABS];
+  frag_t wg[W], wu[W], abuf[KC_SLABS][MT];
   if (wave < nchunks) {
 #pragma unroll
-    for (int s = 0; s < KC_SLABS; ++s) abuf[s] = *reinterpret_cast<const frag_t*>(arow + wave * KC + s * VK_SLAB);
+    for (int mt = 0; mt < MT; ++mt) {
+      const elem_t* arow = act + (int64_t)min(mt * 16 + r16, M - 1) * lda + kg * VK_VEC;
+#pragma unroll
+      for (int s = 0; s < KC_SLABS; ++s) abuf[s][mt] = *reinterpret_cast<const frag_t*>(arow + wave * KC + s * VK_SLAB);
+    }
   }
   auto issue = [&](int tile, int s, int slot) {
     const int64_t row = min(tile * 16 + r16, I - 1);
@@ -281,7 +287,9 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_stream_swiglu_kernel(elem_
   }
   int parity = 0;
   for (; tile < ntiles; tile += gridDim.x) {
-    f32x4 ag = {0.f, 0.f, 0.f, 0.f}, au = {0.f, 0.f, 0.f, 0.f};
+    f32x4 ag[MT], au[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) ag[mt] = au[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
     if (active) {
       const int nt = tile + gridDim.x;
       const bool has_next = nt < ntiles;
@@ -291,17 +299,23 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_stream_swiglu_kernel(elem_
         const frag_t fg = wg[slot], fu = wu[slot];
         if (i + W < KC_SLABS) issue(tile, i + W, slot);
         else if (has_next) issue(nt, i + W - KC_SLABS, slot);
-        ag = mma_slab(fg, abuf[i], ag);
-        au = mma_slab(fu, abuf[i], au);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          ag[mt] = mma_slab(fg, abuf[i][mt], ag[mt]);
+          au[mt] = mma_slab(fu, abuf[i][mt], au[mt]);
+        }
       }
     }
-    part[parity][wave][0][lane] = ag;
-    part[parity][wave][1][lane] = au;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      part[parity][wave][2 * mt][lane] = ag[mt];
+      part[parity][wave][2 * mt + 1][lane] = au[mt];
+    }
     __syncthreads();
-    if (wave == 0) {
+    if (wave < MT) {       // wave mt adds up and finishes the rows of activation tile mt
       f32x4 tg = {0.f, 0.f, 0.f, 0.f}, tu = {0.f, 0.f, 0.f, 0.f};
       for (int w2 = 0; w2 < nchunks; ++w2) {
-        const f32x4 pg = part[parity][w2][0][lane], pu = part[parity][w2][1][lane];
+        const f32x4 pg = part[parity][w2][2 * wave][lane], pu = part[parity][w2][2 * wave + 1][lane];
         tg.x = tg.x + pg.x; tg.y = tg.y + pg.y; tg.z = tg.z + pg.z; tg.w = tg.w + pg.w;
         tu.x = tu.x + pu.x; tu.y = tu.y + pu.y; tu.z = tu.z + pu.z; tu.w = tu.w + pu.w;
       }
@@ -312,7 +326,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_stream_swiglu_kernel(elem_
       y.y = (g[1] * (1.0f / (1.0f + expf(-g[1])))) * u[1];
       y.z = (g[2] * (1.0f / (1.0f + expf(-g[2])))) * u[2];
       y.w = (g[3] * (1.0f / (1.0f + expf(-g[3])))) * u[3];
-      store_out4(out, ldo, r16, tile * 16 + 4 * kg, M, I, y, out_vec_ok);
+      store_out4(out, ldo, wave * 16 + r16, tile * 16 + 4 * kg, M, I, y, out_vec_ok);
     }
     parity ^= 1;
   }
@@ -805,7 +819,8 @@ extern "C" {
 // kernel: 0 = choose by size, 1 = skinny (M <= 64), 2 = tiled (pipelined if K allows), 3 = tiled through
 // registers, 4..6 = pipelined with 2..4 stages, 7 = skinny with two weight tiles per workgroup where it has
 // such a variant, 8, 9 and 10 = activations shared through LDS with 64, 32 and 128 weight rows per workgroup
-// (17 to 64 rows; for measurements and tests).  The result does not depend on the choice.
+// (17 to 64 rows), 11 = skinny with two activation tiles resident in registers (17 to 32 rows of 16-bit
+// elements, K <= 4096); for measurements and tests.  The result does not depend on the choice.
 int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K, int64_t lda, int64_t ldo,
             int kernel, hipStream_t st) {
   VK_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
@@ -814,10 +829,12 @@ int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K
              (long long)lda, VK_VEC);
   VK_REQUIRE(ldo >= N, "gemm: output row stride %lld is smaller than N=%d", (long long)ldo, N);
   VK_REQUIRE(((uintptr_t)act % 16) == 0 && ((uintptr_t)w % 16) == 0, "gemm: operands must be 16-byte aligned");
-  VK_REQUIRE(kernel >= 0 && kernel <= 10, "gemm: unknown kernel %d", kernel);
+  VK_REQUIRE(kernel >= 0 && kernel <= 11, "gemm: unknown kernel %d", kernel);
   if (M == 0) return 0;
   const int vec_ok = (ldo % 4 == 0) && ((uintptr_t)out % 16 == 0);
-  // Measured on Qwen3-8B shapes (MI355X).  Up to 16 rows: the streaming kernel.  17 to 64 rows with K in
+  // Measured on Qwen3-8B shapes (MI355X).  Up to 16 rows: the streaming kernel.  17 to 32 rows of 16-bit
+  // elements with K up to 4096 and 6144 weight rows or more: the streaming kernel with both activation
+  // tiles of a wave's chunk in registers (32 rows, 24576 x 4096: 53 -> 44 us).  Else 17 to 64 rows with K in
   // whole chunks: the kernel that shares activations through LDS: 128 weight rows per workgroup from
   // 24576 weight rows on (the activations that every workgroup reads are then half the weight bytes:
   // 64 rows, 51200 x 5120: 158 -> 127 us), 64 from 16384 on; with fewer, 32 weight rows from 41 rows on, and below
@@ -825,6 +842,7 @@ int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K
   // rows: the pipelined tile kernel.
   if (kernel == 0) {
     if (M <= 16) kernel = 1;
+    else if (M <= 32 && K % KC == 0 && K <= SK_WAVES * KC && N >= 6144 && sizeof(elem_t) == 2) kernel = 11;
     else if (M <= 64 && K % KC == 0) kernel = N >= 24576 ? 10 : (N >= 16384 ? 8 : (M > 40 ? 9 : (N >= 6144 ? 7 : 1)));
     else if (M <= 64) kernel = (N >= 16384 && M > 32) ? 2 : (N >= 6144 ? 7 : 1);
     else kernel = 2;
@@ -846,7 +864,10 @@ int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K
     if (mt == 3) return launch_mid<3, 4>(out, act, w, M, N, K, lda, ldo, vec_ok, st);
     return launch_mid<4, 4>(out, act, w, M, N, K, lda, ldo, vec_ok, st);
   }
-  if (kernel == 1 || kernel == 7) {
+  if (kernel == 11)
+    VK_REQUIRE(M > 16 && M <= 32 && K % KC == 0 && K <= SK_WAVES * KC && sizeof(elem_t) == 2,
+               "gemm: resident activations of two tiles need 17 to 32 rows of 16-bit elements and K a multiple of %d up to %d", KC, SK_WAVES * KC);
+  if (kernel == 1 || kernel == 7 || kernel == 11) {
     VK_REQUIRE(M <= 64, "gemm: the skinny kernel takes at most 64 rows, got %d", M);
     const int mt = (M + 15) / 16;
     const unsigned grid = (unsigned)((N + 15) / 16);
@@ -867,7 +888,14 @@ int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K
                                          64 * SK_WAVES, 0, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok); \
   } while (0)
       if (mt == 1) { if (K <= SK_WAVES * KC) ST(1, 8, true, 1); else ST(1, 8, false, 1); }
-      else if (mt == 2) { if (kernel == 7) ST(2, 4, false, 2); else ST(2, 8, false, 1); }
+      else if (mt == 2) {
+#ifdef VK_BF16
+        if (kernel == 11) ST(2, 8, true, 1);
+        else
+#endif
+        if (kernel == 7) ST(2, 4, false, 2);
+        else ST(2, 8, false, 1);
+      }
       else if (mt == 3) { if (kernel == 7) ST(3, 4, false, 2); else ST(3, 4, false, 1); }
       else { if (kernel == 7) ST(4, 4, false, 2); else ST(4, 4, false, 1); }
 #undef ST
@@ -896,6 +924,9 @@ int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K
 // 1: the streaming kernel (few rows), 2: the pipelined tile kernel (many rows), 0: neither.
 int vk_gemm_swiglu_supported(int M, int I, int K) {
   if (M >= 1 && M <= 16 && I > 0 && K % KC == 0 && K <= SK_WAVES * KC) return 1;
+#ifdef VK_BF16
+  if (M > 16 && M <= 32 && I > 0 && K % KC == 0 && K <= SK_WAVES * KC) return 1;    // two activation tiles in registers
+#endif
   if (M > 64 && I > 0 && K % (2 * VK_SLAB) == 0) return 2;
   return 0;
 }
@@ -909,18 +940,28 @@ int vk_gemm_swiglu(elem_t* out, const elem_t* act, const elem_t* w, int M, int I
   VK_REQUIRE(((uintptr_t)act % 16) == 0 && ((uintptr_t)w % 16) == 0, "gemm_swiglu: operands must be 16-byte aligned");
   if (how == 2)
     return launch_pipe<2, true>(out, act, w, M, I, K, lda, ldo, (ldo % 4 == 0) && ((uintptr_t)out % 16 == 0), st);
-  static int resident = 0;
-  if (resident == 0) {
-    int dev = 0, cus = 0, per_cu = 0;
-    (void)hipGetDevice(&dev);
-    (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-    (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gemm_stream_swiglu_kernel<8>, 64 * SK_WAVES, 0);
-    resident = (cus > 0 ? cus : 256) * (per_cu > 0 ? per_cu : 1);
-  }
   const int ntiles = (I + 15) / 16;
   const int vec_ok = (ldo % 4 == 0) && ((uintptr_t)out % 16 == 0);
-  gemm_stream_swiglu_kernel<8><<<ntiles < resident ? ntiles : resident, 64 * SK_WAVES, 0, st>>>(out, act, w, M, I, K,
-                                                                                               lda, ldo, vec_ok);
+#define SWIGLU_STREAM(W, MT)                                                                               \
+  do {                                                                                                     \
+    static int resident = 0;                                                                               \
+    if (resident == 0) {                                                                                   \
+      int dev = 0, cus = 0, per_cu = 0;                                                                    \
+      (void)hipGetDevice(&dev);                                                                            \
+      (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);                       \
+      (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gemm_stream_swiglu_kernel<W, MT>,        \
+                                                         64 * SK_WAVES, 0);                                \
+      resident = (cus > 0 ? cus : 256) * (per_cu > 0 ? per_cu : 1);                                        \
+    }                                                                                                      \
+    gemm_stream_swiglu_kernel<W, MT><<<ntiles < resident ? ntiles : resident, 64 * SK_WAVES, 0, st>>>(     \
+        out, act, w, M, I, K, lda, ldo, vec_ok);                                                           \
+  } while (0)
+#ifdef VK_BF16
+  if (M > 16) SWIGLU_STREAM(4, 2);
+  else
+#endif
+    SWIGLU_STREAM(8, 1);
+#undef SWIGLU_STREAM
   return vk_check_launch("gemm_swiglu");
 }
 
