@@ -138,10 +138,10 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_kernel(elem_t* __re
 // a wave's window of W slabs in flight runs on across tile borders, so the
 // memory pipe never drains; no load is predicated (rows beyond N or M are
 // clamped to the last valid row and their results dropped), because a select on
-// a loaded value makes the compiler wait for it at once; and with RES (K <= 4096,
-// one 16-row activation tile) a wave keeps the activations of its chunk in
-// registers for the whole kernel.  One barrier per round of eight chunks.
-template <int MT, int W, bool RES, int NT>
+// a loaded value makes the compiler wait for it at once; and with RC > 0 a wave
+// keeps the activations of its RC chunks (K <= RC * 4096) in registers for the
+// whole kernel.  One barrier per round of eight chunks.
+template <int MT, int W, int RC, int NT>
 __global__ __launch_bounds__(64 * SK_WAVES) void gemm_stream_kernel(elem_t* __restrict__ out,
                                                                     const elem_t* __restrict__ act,
                                                                     const elem_t* __restrict__ w, int M, int N, int K,
@@ -150,7 +150,10 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_stream_kernel(elem_t* __re
   // activations once, M * K elements beside its 16 * NT * K weights: more weight rows per workgroup
   // keep that traffic, which comes from the second-level cache, in proportion.
   static_assert(KC_SLABS % W == 0, "the window must divide a chunk");
-  static_assert(!RES || MT <= 2, "resident activations are for one or two activation tiles");
+  // RC: chunks per wave whose activations stay in registers for the whole kernel (0: none are kept;
+  // K <= RC * 8 chunks).  A chunk of one activation tile is 64 registers of 16-bit elements.
+  constexpr bool RES = RC > 0;
+  static_assert(RC * MT <= 2, "resident activations: at most two chunk tiles per wave");
   static_assert(NT * MT <= SK_WAVES, "one wave adds up each output tile");
   __shared__ f32x4 part[2][SK_WAVES][NT * MT][64];
 
@@ -163,13 +166,16 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_stream_kernel(elem_t* __re
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) arow[mt] = act + (int64_t)min(mt * 16 + r16, M - 1) * lda + kg * VK_VEC;
 
-  frag_t wbuf[W][NT], abuf[RES ? KC_SLABS : W][MT];
+  frag_t wbuf[W][NT], abuf[RES ? RC * KC_SLABS : W][MT];
   if (RES) {
-    if (wave < nchunks) {
+#pragma unroll
+    for (int r = 0; r < RC; ++r) {
+      const int c = min(r * SK_WAVES + wave, nchunks - 1);     // beyond K: the last chunk again (not used)
 #pragma unroll
       for (int s = 0; s < KC_SLABS; ++s)
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) abuf[s][mt] = *reinterpret_cast<const frag_t*>(arow[mt] + wave * KC + s * VK_SLAB);
+        for (int mt = 0; mt < MT; ++mt)
+          abuf[r * KC_SLABS + s][mt] = *reinterpret_cast<const frag_t*>(arow[mt] + c * KC + s * VK_SLAB);
     }
   }
   auto issue = [&](int tile, int c, int s, int slot) {
@@ -191,7 +197,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_stream_kernel(elem_t* __re
   int parity = 0;
   for (; tile < ntiles; tile += gridDim.x) {
     f32x4 total = {0.f, 0.f, 0.f, 0.f};
-    for (int base = 0; base < nchunks; base += SK_WAVES) {
+    auto round = [&](int base, int r) {       // chunks base .. base + 7; r = base / 8 where that is a constant
       const int c = base + wave;
       f32x4 acc[NT][MT];
 #pragma unroll
@@ -213,7 +219,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_stream_kernel(elem_t* __re
 #pragma unroll
           for (int nt = 0; nt < NT; ++nt) fw[nt] = wbuf[slot][nt];
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt) fa[mt] = RES ? abuf[i][mt] : abuf[slot][mt];
+          for (int mt = 0; mt < MT; ++mt) fa[mt] = RES ? abuf[r * KC_SLABS + i][mt] : abuf[slot][mt];
           if (i + W < KC_SLABS) issue(tile, c, i + W, slot);
           else if (has_next) issue(nt_, nc, i + W - KC_SLABS, slot);
 #pragma unroll
@@ -236,6 +242,13 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_stream_kernel(elem_t* __re
         }
       }
       parity ^= 1;
+    };
+    if (RES) {
+#pragma unroll
+      for (int r = 0; r < (RES ? RC : 1); ++r)
+        if (r * SK_WAVES < nchunks) round(r * SK_WAVES, r);
+    } else {
+      for (int base = 0; base < nchunks; base += SK_WAVES) round(base, 0);
     }
     if (wave < NT * MT)
       store_out4(out, ldo, (wave % MT) * 16 + r16, (tile * NT + wave / MT) * 16 + 4 * kg, M, N, total, out_vec_ok);
@@ -248,74 +261,87 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_stream_kernel(elem_t* __re
 // two projections rounded to the element type first, which is what the separate
 // GEMM and SwiGLU kernels compute (kernels/triton_kernels/silu_mul.py:64-87).
 // M <= 16, K <= 4096 (activations resident in registers).
-template <int W, int MT>
+template <int W, int MT, int RC>
 __global__ __launch_bounds__(64 * SK_WAVES) void gemm_stream_swiglu_kernel(elem_t* __restrict__ out,
                                                                            const elem_t* __restrict__ act,
                                                                            const elem_t* __restrict__ w, int M, int I,
                                                                            int K, int64_t lda, int64_t ldo,
                                                                            int out_vec_ok) {
   static_assert(KC_SLABS % W == 0, "the window must divide a chunk");
-  static_assert(MT <= 2, "one or two activation tiles stay in registers");
-  __shared__ f32x4 part[2][SK_WAVES][2 * MT][64];
+  static_assert(MT * RC <= 2, "two chunk tiles of activations stay in registers: two tiles of a chunk or two chunks of a tile");
+  __shared__ f32x4 part[2][RC][SK_WAVES][2 * MT][64];      // two sets, used in turn: one barrier per tile
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r16 = lane & 15, kg = lane >> 4;
   const int nchunks = K / KC;
   const int ntiles = (I + 15) / 16;
 
-  frag_t wg[W], wu[W], abuf[KC_SLABS][MT];
-  if (wave < nchunks) {
+  // Wave w has chunks w, w + 8, ...: RC of them (chunks beyond K are read as the last and not used).
+  frag_t wg[W], wu[W], abuf[RC * KC_SLABS][MT];
+#pragma unroll
+  for (int r = 0; r < RC; ++r) {
+    const int c = min(r * SK_WAVES + wave, nchunks - 1);
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       const elem_t* arow = act + (int64_t)min(mt * 16 + r16, M - 1) * lda + kg * VK_VEC;
 #pragma unroll
-      for (int s = 0; s < KC_SLABS; ++s) abuf[s][mt] = *reinterpret_cast<const frag_t*>(arow + wave * KC + s * VK_SLAB);
+      for (int s = 0; s < KC_SLABS; ++s)
+        abuf[r * KC_SLABS + s][mt] = *reinterpret_cast<const frag_t*>(arow + c * KC + s * VK_SLAB);
     }
   }
-  auto issue = [&](int tile, int s, int slot) {
+  // Slab g of this wave's stream over a tile: chunk (g / 16) * 8 + wave, slab g % 16 of it.
+  const int my_chunks = wave < nchunks ? (nchunks - wave + SK_WAVES - 1) / SK_WAVES : 0;     // <= RC
+  const int my_slabs = my_chunks * KC_SLABS;
+  auto issue = [&](int tile, int g, int slot) {
     const int64_t row = min(tile * 16 + r16, I - 1);
-    const elem_t* p = w + row * K + kg * VK_VEC + wave * KC + s * VK_SLAB;
+    const int c = (g / KC_SLABS) * SK_WAVES + wave;
+    const elem_t* p = w + row * K + kg * VK_VEC + (int64_t)c * KC + (g % KC_SLABS) * VK_SLAB;
     wg[slot] = *reinterpret_cast<const frag_t*>(p);
     wu[slot] = *reinterpret_cast<const frag_t*>(p + (int64_t)I * K);
   };
 
   int tile = blockIdx.x;
-  const bool active = wave < nchunks;
+  const bool active = my_chunks > 0;
   if (tile < ntiles && active) {
 #pragma unroll
     for (int i = 0; i < W; ++i) issue(tile, i, i);
   }
   int parity = 0;
   for (; tile < ntiles; tile += gridDim.x) {
-    f32x4 ag[MT], au[MT];
+    const int nt = tile + gridDim.x;
+    const bool has_next = nt < ntiles;
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) ag[mt] = au[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-    if (active) {
-      const int nt = tile + gridDim.x;
-      const bool has_next = nt < ntiles;
+    for (int r = 0; r < RC; ++r) {
+      f32x4 ag[MT], au[MT];
 #pragma unroll
-      for (int i = 0; i < KC_SLABS; ++i) {
-        const int slot = i % W;
-        const frag_t fg = wg[slot], fu = wu[slot];
-        if (i + W < KC_SLABS) issue(tile, i + W, slot);
-        else if (has_next) issue(nt, i + W - KC_SLABS, slot);
+      for (int mt = 0; mt < MT; ++mt) ag[mt] = au[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (r < my_chunks) {
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          ag[mt] = mma_slab(fg, abuf[i][mt], ag[mt]);
-          au[mt] = mma_slab(fu, abuf[i][mt], au[mt]);
+        for (int i = 0; i < KC_SLABS; ++i) {
+          const int slot = i % W;
+          const frag_t fg = wg[slot], fu = wu[slot];
+          const int g = r * KC_SLABS + i + W;             // the slab that takes this slot
+          if (g < my_slabs) issue(tile, g, slot);
+          else if (has_next) issue(nt, g - my_slabs, slot);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            ag[mt] = mma_slab(fg, abuf[r * KC_SLABS + i][mt], ag[mt]);
+            au[mt] = mma_slab(fu, abuf[r * KC_SLABS + i][mt], au[mt]);
+          }
         }
       }
-    }
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      part[parity][wave][2 * mt][lane] = ag[mt];
-      part[parity][wave][2 * mt + 1][lane] = au[mt];
+      for (int mt = 0; mt < MT; ++mt) {
+        part[parity][r][wave][2 * mt][lane] = ag[mt];
+        part[parity][r][wave][2 * mt + 1][lane] = au[mt];
+      }
     }
     __syncthreads();
-    if (wave < MT) {       // wave mt adds up and finishes the rows of activation tile mt
+    if (wave < MT) {       // wave mt adds up, in chunk order, and finishes the rows of activation tile mt
       f32x4 tg = {0.f, 0.f, 0.f, 0.f}, tu = {0.f, 0.f, 0.f, 0.f};
-      for (int w2 = 0; w2 < nchunks; ++w2) {
-        const f32x4 pg = part[parity][w2][2 * wave][lane], pu = part[parity][w2][2 * wave + 1][lane];
+      for (int c = 0; c < nchunks; ++c) {
+        const f32x4 pg = part[parity][c / SK_WAVES][c % SK_WAVES][2 * wave][lane];
+        const f32x4 pu = part[parity][c / SK_WAVES][c % SK_WAVES][2 * wave + 1][lane];
         tg.x = tg.x + pg.x; tg.y = tg.y + pg.y; tg.z = tg.z + pg.z; tg.w = tg.w + pg.w;
         tu.x = tu.x + pu.x; tu.y = tu.y + pu.y; tu.z = tu.z + pu.z; tu.w = tu.w + pu.w;
       }
@@ -872,32 +898,40 @@ int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K
     const int mt = (M + 15) / 16;
     const unsigned grid = (unsigned)((N + 15) / 16);
     if (K % KC == 0) {
-#define ST(MT, W, RES, NT)                                                                                \
+#define ST(MT, W, RC, NT)                                                                                 \
   do {                                                                                                    \
     static int resident = 0; /* workgroups of this kernel that the device holds at once */               \
     if (resident == 0) {                                                                                  \
       int dev = 0, cus = 0, per_cu = 0;                                                                   \
       (void)hipGetDevice(&dev);                                                                           \
       (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);                      \
-      (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gemm_stream_kernel<MT, W, RES, NT>,     \
+      (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gemm_stream_kernel<MT, W, RC, NT>,      \
                                                          64 * SK_WAVES, 0);                               \
       resident = (cus > 0 ? cus : 256) * (per_cu > 0 ? per_cu : 1);                                       \
     }                                                                                                     \
     const unsigned groups = (unsigned)((N + 16 * NT - 1) / (16 * NT));                                    \
-    gemm_stream_kernel<MT, W, RES, NT><<<groups < (unsigned)resident ? groups : (unsigned)resident,       \
+    gemm_stream_kernel<MT, W, RC, NT><<<groups < (unsigned)resident ? groups : (unsigned)resident,        \
                                          64 * SK_WAVES, 0, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok); \
   } while (0)
-      if (mt == 1) { if (K <= SK_WAVES * KC) ST(1, 8, true, 1); else ST(1, 8, false, 1); }
+      if (mt == 1) {
+        if (K <= SK_WAVES * KC) ST(1, 8, 1, 1);
+#ifdef VK_BF16
+        // Two chunks a wave are 128 registers of activations (16 rows, 34816 x 5120: 118 -> 87 us);
+        // three did not fit beside the rest and were slower than none (4096 x 12288: 29 -> 36 us).
+        else if (K <= 2 * SK_WAVES * KC) ST(1, 8, 2, 1);
+#endif
+        else ST(1, 8, 0, 1);
+      }
       else if (mt == 2) {
 #ifdef VK_BF16
-        if (kernel == 11) ST(2, 8, true, 1);
+        if (kernel == 11) ST(2, 8, 1, 1);
         else
 #endif
-        if (kernel == 7) ST(2, 4, false, 2);
-        else ST(2, 8, false, 1);
+        if (kernel == 7) ST(2, 4, 0, 2);
+        else ST(2, 8, 0, 1);
       }
-      else if (mt == 3) { if (kernel == 7) ST(3, 4, false, 2); else ST(3, 4, false, 1); }
-      else { if (kernel == 7) ST(4, 4, false, 2); else ST(4, 4, false, 1); }
+      else if (mt == 3) { if (kernel == 7) ST(3, 4, 0, 2); else ST(3, 4, 0, 1); }
+      else { if (kernel == 7) ST(4, 4, 0, 2); else ST(4, 4, 0, 1); }
 #undef ST
       return vk_check_launch("gemm_stream");
     }
@@ -926,6 +960,7 @@ int vk_gemm_swiglu_supported(int M, int I, int K) {
   if (M >= 1 && M <= 16 && I > 0 && K % KC == 0 && K <= SK_WAVES * KC) return 1;
 #ifdef VK_BF16
   if (M > 16 && M <= 32 && I > 0 && K % KC == 0 && K <= SK_WAVES * KC) return 1;    // two activation tiles in registers
+  if (M >= 1 && M <= 16 && I > 0 && K % KC == 0 && K <= 2 * SK_WAVES * KC) return 1;   // two chunks a wave
 #endif
   if (M > 64 && I > 0 && K % (2 * VK_SLAB) == 0) return 2;
   return 0;
@@ -942,25 +977,26 @@ int vk_gemm_swiglu(elem_t* out, const elem_t* act, const elem_t* w, int M, int I
     return launch_pipe<2, true>(out, act, w, M, I, K, lda, ldo, (ldo % 4 == 0) && ((uintptr_t)out % 16 == 0), st);
   const int ntiles = (I + 15) / 16;
   const int vec_ok = (ldo % 4 == 0) && ((uintptr_t)out % 16 == 0);
-#define SWIGLU_STREAM(W, MT)                                                                               \
+#define SWIGLU_STREAM(W, MT, RC)                                                                            \
   do {                                                                                                     \
     static int resident = 0;                                                                               \
     if (resident == 0) {                                                                                   \
       int dev = 0, cus = 0, per_cu = 0;                                                                    \
       (void)hipGetDevice(&dev);                                                                            \
       (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);                       \
-      (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gemm_stream_swiglu_kernel<W, MT>,        \
+      (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gemm_stream_swiglu_kernel<W, MT, RC>,    \
                                                          64 * SK_WAVES, 0);                                \
       resident = (cus > 0 ? cus : 256) * (per_cu > 0 ? per_cu : 1);                                        \
     }                                                                                                      \
-    gemm_stream_swiglu_kernel<W, MT><<<ntiles < resident ? ntiles : resident, 64 * SK_WAVES, 0, st>>>(     \
+    gemm_stream_swiglu_kernel<W, MT, RC><<<ntiles < resident ? ntiles : resident, 64 * SK_WAVES, 0, st>>>( \
         out, act, w, M, I, K, lda, ldo, vec_ok);                                                           \
   } while (0)
 #ifdef VK_BF16
-  if (M > 16) SWIGLU_STREAM(4, 2);
+  if (M > 16) SWIGLU_STREAM(4, 2, 1);
+  else if (K > SK_WAVES * KC) SWIGLU_STREAM(4, 1, 2);
   else
 #endif
-    SWIGLU_STREAM(8, 1);
+    SWIGLU_STREAM(8, 1, 1);
 #undef SWIGLU_STREAM
   return vk_check_launch("gemm_swiglu");
 }
