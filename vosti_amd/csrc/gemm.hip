@@ -866,6 +866,7 @@ int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K
   // 64 rows, 51200 x 5120: 158 -> 127 us), 64 from 16384 on; with fewer, 32 weight rows from 41 rows on, and below
   // that the streaming kernel, with two weight tiles per workgroup from 6144 weight rows on.  More
   // rows: the pipelined tile kernel.
+  const bool by_size = kernel == 0;
   if (kernel == 0) {
     if (M <= 16) kernel = 1;
     else if (M <= 32 && K % KC == 0 && K <= SK_WAVES * KC && N >= 6144 && sizeof(elem_t) == 2) kernel = 11;
@@ -914,7 +915,19 @@ int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K
                                          64 * SK_WAVES, 0, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok); \
   } while (0)
       if (mt == 1) {
-        if (K <= SK_WAVES * KC) ST(1, 8, 1, 1);
+        // A few weight tiles more than workgroups in flight (one per compute unit) would mean a second
+        // pass of a few: two tiles a workgroup then finish sooner (16 rows, 5120 x 25600: 111 -> 86 us),
+        // unless one chunk a wave keeps the activations in registers (6144 x 4096: 12.6 against 15.7 us).
+        static int cus = 0;
+        if (cus == 0) {
+          int dev = 0;
+          (void)hipGetDevice(&dev);
+          (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+          if (cus <= 0) cus = 256;
+        }
+        const int tiles16 = (N + 15) / 16;
+        if (kernel == 7 || (by_size && K > SK_WAVES * KC && tiles16 > cus && 2 * tiles16 <= 3 * cus)) ST(1, 8, 0, 2);
+        else if (K <= SK_WAVES * KC) ST(1, 8, 1, 1);
 #ifdef VK_BF16
         // Two chunks a wave are 128 registers of activations (16 rows, 34816 x 5120: 118 -> 87 us);
         // three did not fit beside the rest and were slower than none (4096 x 12288: 29 -> 36 us).
