@@ -699,10 +699,14 @@ __device__ __forceinline__ void mid_load_to_lds16(const elem_t* src, unsigned ch
   __builtin_amdgcn_global_load_lds(src, (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
 }
 
-template <int MT, int KH>
+// SWIGLU (one chunk in work, KH = 1): w holds N gate rows, then N up rows; waves 0..3 take four gate
+// tiles, waves 4..7 the matching up tiles, and out[m, n] = silu(g) * u with g and u rounded to the
+// element type first, as the separate kernels compute it.
+template <int MT, int KH, bool SWIGLU = false>
 __global__ __launch_bounds__(512) void gemm_mid_kernel(elem_t* __restrict__ out, const elem_t* __restrict__ act,
                                                        const elem_t* __restrict__ w, int M, int N, int K,
                                                        int64_t lda, int64_t ldo, int out_vec_ok) {
+  static_assert(!SWIGLU || KH == 1, "the SwiGLU epilogue pairs the waves of one chunk");
   constexpr int NTW = 8 / KH;                       // weight tiles of the workgroup (16 rows each)
   constexpr int STEPS = KC_SLABS / MID_QS;          // steps per chunk
   constexpr int ROW_B = MID_QS * 64;                // bytes of an activation row in a step: 256
@@ -722,7 +726,9 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(elem_t* __restrict__ out,
 
   // Weights: row of this wave's tile, chunk sequence kh, kh + KH, ...; a chunk beyond the last is read as
   // the last (and not used), so that every wave issues the same number of loads.
-  const elem_t* wrow = w + (int64_t)min((int)blockIdx.x * 16 * NTW + nt * 16 + r16, N - 1) * K + kg * VK_VEC;
+  const int out_col0 = SWIGLU ? (int)blockIdx.x * 64 + (nt & 3) * 16 : (int)blockIdx.x * 16 * NTW + nt * 16;
+  const int64_t wrow_i = SWIGLU ? (int64_t)(nt >> 2) * N + min(out_col0 + r16, N - 1) : min(out_col0 + r16, N - 1);
+  const elem_t* wrow = w + wrow_i * K + kg * VK_VEC;
   frag_t wbuf[MID_W];
   auto issue_w = [&](int g, int slot) {              // g: this wave's slab number; slot = g % MID_W
     const int gg = min(g, nsteps * MID_QS - 1);
@@ -819,23 +825,51 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(elem_t* __restrict__ out,
   mid_barrier();
   if (kh == 0) {
     close_group(last_full);
+    if (SWIGLU) {
+      // Every wave is past the barrier above, so the activation buffers are free: the up waves leave
+      // their sums there for the gate waves of the same columns.
+      f32x4* ex = reinterpret_cast<f32x4*>(lds);       // [4 tiles][MT][64 lanes]
+      if (nt >= 4) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) ex[((nt - 4) * MT + mt) * 64 + lane] = total[mt];
+      }
+      __syncthreads();
+      if (nt < 4) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          const f32x4 t = total[mt], o = ex[(nt * MT + mt) * 64 + lane];
+          const float g[4] = {round_to_elem(t.x), round_to_elem(t.y), round_to_elem(t.z), round_to_elem(t.w)};
+          const float u[4] = {round_to_elem(o.x), round_to_elem(o.y), round_to_elem(o.z), round_to_elem(o.w)};
+          f32x4 y;
+          y.x = (g[0] * (1.0f / (1.0f + expf(-g[0])))) * u[0];
+          y.y = (g[1] * (1.0f / (1.0f + expf(-g[1])))) * u[1];
+          y.z = (g[2] * (1.0f / (1.0f + expf(-g[2])))) * u[2];
+          y.w = (g[3] * (1.0f / (1.0f + expf(-g[3])))) * u[3];
+          store_out4(out, ldo, mt * 16 + r16, out_col0 + 4 * kg, M, N, y, out_vec_ok);
+        }
+      }
+      return;
+    }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
-      store_out4(out, ldo, mt * 16 + r16, blockIdx.x * 16 * NTW + nt * 16 + 4 * kg, M, N, total[mt], out_vec_ok);
+      store_out4(out, ldo, mt * 16 + r16, out_col0 + 4 * kg, M, N, total[mt], out_vec_ok);
   }
 }
 
-template <int MT, int KH>
+// N: weight rows, or with SWIGLU the gate rows (and as many up rows after them).
+template <int MT, int KH, bool SWIGLU = false>
 static int launch_mid(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K, int64_t lda, int64_t ldo,
                       int vec_ok, hipStream_t st) {
   constexpr int NTW = 8 / KH;
+  constexpr int COLS = SWIGLU ? 64 : 16 * NTW;      // output columns of a workgroup
   const size_t smem = (size_t)2 * KH * 16 * MT * (MID_QS * 64) + (size_t)(KH - 1) * NTW * MT * 64 * sizeof(f32x4);
+  static_assert(!SWIGLU || 2 * 16 * MT * (MID_QS * 64) >= 4 * MT * 64 * (int)sizeof(f32x4), "the exchange fits the activation buffers");
   static bool configured = false;
   if (!configured) {
-    (void)hipFuncSetAttribute((const void*)gemm_mid_kernel<MT, KH>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    (void)hipFuncSetAttribute((const void*)gemm_mid_kernel<MT, KH, SWIGLU>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     configured = true;
   }
-  gemm_mid_kernel<MT, KH><<<(N + 16 * NTW - 1) / (16 * NTW), 512, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok);
+  gemm_mid_kernel<MT, KH, SWIGLU><<<(N + COLS - 1) / COLS, 512, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok);
   return vk_check_launch("gemm_mid");
 }
 
@@ -968,7 +1002,8 @@ int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K
 }
 
 // 1 if vk_gemm_swiglu takes these sizes (the caller otherwise runs vk_gemm and vk_swiglu, with the same result).
-// 1: the streaming kernel (few rows), 2: the pipelined tile kernel (many rows), 0: neither.
+// 1: the streaming kernel (few rows), 2: the pipelined tile kernel (many rows), 3: the kernel for 17 to 64
+// rows that shares activations through LDS, 0: none.
 int vk_gemm_swiglu_supported(int M, int I, int K) {
   if (M >= 1 && M <= 16 && I > 0 && K % KC == 0 && K <= SK_WAVES * KC) return 1;
 #ifdef VK_BF16
@@ -976,6 +1011,7 @@ int vk_gemm_swiglu_supported(int M, int I, int K) {
   if (M >= 1 && M <= 16 && I > 0 && K % KC == 0 && K <= 2 * SK_WAVES * KC) return 1;   // two chunks a wave
 #endif
   if (M > 64 && I > 0 && K % (2 * VK_SLAB) == 0) return 2;
+  if (M > 16 && M <= 64 && I > 0 && K % KC == 0) return 3;      // activations shared through LDS
   return 0;
 }
 
@@ -988,6 +1024,11 @@ int vk_gemm_swiglu(elem_t* out, const elem_t* act, const elem_t* w, int M, int I
   VK_REQUIRE(((uintptr_t)act % 16) == 0 && ((uintptr_t)w % 16) == 0, "gemm_swiglu: operands must be 16-byte aligned");
   if (how == 2)
     return launch_pipe<2, true>(out, act, w, M, I, K, lda, ldo, (ldo % 4 == 0) && ((uintptr_t)out % 16 == 0), st);
+  if (how == 3) {
+    const int ok4 = (ldo % 4 == 0) && ((uintptr_t)out % 16 == 0);
+    if (M <= 32) return launch_mid<2, 1, true>(out, act, w, M, I, K, lda, ldo, ok4, st);
+    return launch_mid<4, 1, true>(out, act, w, M, I, K, lda, ldo, ok4, st);
+  }
   const int ntiles = (I + 15) / 16;
   const int vec_ok = (ldo % 4 == 0) && ((uintptr_t)out % 16 == 0);
 #define SWIGLU_STREAM(W, MT, RC)                                                                            \
