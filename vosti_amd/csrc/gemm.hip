@@ -874,6 +874,17 @@ static int launch_mid(elem_t* out, const elem_t* act, const elem_t* w, int M, in
 }
 
 // ==================================================================== host
+static int device_cus() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (cus <= 0) cus = 256;
+  }
+  return cus;
+}
+
 extern "C" {
 
 // kernel: 0 = choose by size, 1 = skinny (M <= 64), 2 = tiled (pipelined if K allows), 3 = tiled through
@@ -897,14 +908,22 @@ int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K
   // tiles of a wave's chunk in registers (32 rows, 24576 x 4096: 53 -> 44 us).  Else 17 to 64 rows with K in
   // whole chunks: the kernel that shares activations through LDS: 128 weight rows per workgroup from
   // 24576 weight rows on (the activations that every workgroup reads are then half the weight bytes:
-  // 64 rows, 51200 x 5120: 158 -> 127 us), 64 from 16384 on; with fewer, 32 weight rows from 41 rows on, and below
+  // 64 rows, 51200 x 5120: 158 -> 127 us), 64 from 8192 on; with fewer, 32 weight rows from 41 rows on, or
+  // when K is over 4096 and there are more 16-row weight tiles than compute units, so that the streaming
+  // kernel would need a second pass for a few of them (32 rows, 5120 x 17408: 111 -> 65 us); and below
   // that the streaming kernel, with two weight tiles per workgroup from 6144 weight rows on.  More
   // rows: the pipelined tile kernel.
   const bool by_size = kernel == 0;
   if (kernel == 0) {
     if (M <= 16) kernel = 1;
     else if (M <= 32 && K % KC == 0 && K <= SK_WAVES * KC && N >= 6144 && sizeof(elem_t) == 2) kernel = 11;
-    else if (M <= 64 && K % KC == 0) kernel = N >= 24576 ? 10 : (N >= 16384 ? 8 : (M > 40 ? 9 : (N >= 6144 ? 7 : 1)));
+    else if (M <= 64 && K % KC == 0) {
+      if (N >= 24576) kernel = 10;
+      else if (N >= 8192) kernel = 8;
+      else if (M > 40) kernel = 9;
+      else if (K <= SK_WAVES * KC || (N + 15) / 16 <= device_cus()) kernel = N >= 6144 ? 7 : 1;
+      else kernel = 9;
+    }
     else if (M <= 64) kernel = (N >= 16384 && M > 32) ? 2 : (N >= 6144 ? 7 : 1);
     else kernel = 2;
   }
@@ -952,13 +971,7 @@ int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K
         // A few weight tiles more than workgroups in flight (one per compute unit) would mean a second
         // pass of a few: two tiles a workgroup then finish sooner (16 rows, 5120 x 25600: 111 -> 86 us),
         // unless one chunk a wave keeps the activations in registers (6144 x 4096: 12.6 against 15.7 us).
-        static int cus = 0;
-        if (cus == 0) {
-          int dev = 0;
-          (void)hipGetDevice(&dev);
-          (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-          if (cus <= 0) cus = 256;
-        }
+        const int cus = device_cus();
         const int tiles16 = (N + 15) / 16;
         if (kernel == 7 || (by_size && K > SK_WAVES * KC && tiles16 > cus && 2 * tiles16 <= 3 * cus)) ST(1, 8, 0, 2);
         else if (K <= SK_WAVES * KC) ST(1, 8, 1, 1);
