@@ -31,17 +31,21 @@ def rand(shape, dtype, seed, scale=1.0):
 @pytest.mark.parametrize("M,N,K", [(1, 64, 64), (5, 503, 96), (17, 224, 96), (64, 256, 224), (16, 48, 520),
                                    (65, 130, 520), (130, 96, 1032), (300, 520, 2056), (8, 40, 4104),
                                    (8, 4100, 1024), (3, 72, 512), (33, 200, 1536), (64, 4096, 4608), (17, 90, 5120),
-                                   (40, 6200, 1024), (64, 6144, 512), (23, 24, 2048), (48, 24700, 512), (20, 24576, 1024), (31, 6200, 4096), (17, 100, 1536), (9, 130, 12288), (16, 72, 8704), (2, 40, 5120)])
+                                   (40, 6200, 1024), (64, 6144, 512), (23, 24, 2048), (48, 24700, 512), (20, 24576, 1024), (31, 6200, 4096), (17, 100, 1536), (9, 130, 12288), (16, 72, 8704), (2, 40, 5120), (100, 200, 1024), (65, 4100, 512), (130, 96, 1536),
+                                   (250, 8200, 512), (129, 300, 4608)])
 def test_gemm(dtype, M, N, K):
     k = kern(dtype)
     a, w = rand((M, K), dtype, 1), rand((N, K), dtype, 2, 0.1)
     ref = (a.double() @ w.double().t()).float()
     got_t = k.gemm(a.cuda(), w.cuda(), kernel=2)
     torch.testing.assert_close(got_t.float().cpu(), ref.to(dtype).float(), **tol(dtype))
+    if 64 < M <= 512 and K % 512 == 0:
+        for code in (0, 8, 9, 10, 12):  # blocks of 64 (12: of 32) rows through the kernels that share activations through LDS
+            assert torch.equal(k.gemm(a.cuda(), w.cuda(), kernel=code), got_t), code
     if M <= 64:
         codes = [1, 7, 0]           # one and two weight tiles per workgroup, and the kernel chosen by size
         if M > 16 and K % 512 == 0:
-            codes += [8, 9, 10]     # activations shared through LDS: two, four and one chunk in work
+            codes += [8, 9, 10, 12] # activations shared through LDS: two, four and one chunk in work; 12: blocks of 32 rows
         if 16 < M <= 32 and K % 512 == 0 and K <= 4096 and dtype == torch.bfloat16:
             codes += [11]           # two activation tiles resident in registers
         for code in codes:

@@ -720,6 +720,7 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(elem_t* __restrict__ out,
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r16 = lane & 15, kg = lane >> 4;
   const int nt = wave % NTW, kh = wave / NTW;
+  const int row0 = blockIdx.y * 16 * MT;            // more than 16 MT rows: one block of them per blockIdx.y
   const int nchunks = K / KC, ngroups = (nchunks + KH - 1) / KH;     // group: KH chunks in work together
   const int nsteps = ngroups * STEPS;
   const int last_full = nchunks - (ngroups - 1) * KH;                // chunks of the last group: 1 .. KH
@@ -744,7 +745,7 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(elem_t* __restrict__ out,
     const int id = wave * DMA + j;                   // 0 .. 4 MT KH - 1
     const int h = id / (4 * MT), row = (id % (4 * MT)) * 4 + (lane >> 4);
     ah[j] = h;
-    asrc[j] = act + (int64_t)min(row, M - 1) * lda + (((lane & 15) ^ (row & 15)) * VK_VEC);
+    asrc[j] = act + (int64_t)min(row0 + row, M - 1) * lda + (((lane & 15) ^ (row & 15)) * VK_VEC);
     adst[j] = h * HALF_B + (id % (4 * MT)) * 4 * ROW_B;
   }
   auto issue_a = [&](int t) {                        // step t of the workgroup
@@ -845,14 +846,14 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(elem_t* __restrict__ out,
           y.y = (g[1] * (1.0f / (1.0f + expf(-g[1])))) * u[1];
           y.z = (g[2] * (1.0f / (1.0f + expf(-g[2])))) * u[2];
           y.w = (g[3] * (1.0f / (1.0f + expf(-g[3])))) * u[3];
-          store_out4(out, ldo, mt * 16 + r16, out_col0 + 4 * kg, M, N, y, out_vec_ok);
+          store_out4(out, ldo, row0 + mt * 16 + r16, out_col0 + 4 * kg, M, N, y, out_vec_ok);
         }
       }
       return;
     }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
-      store_out4(out, ldo, mt * 16 + r16, out_col0 + 4 * kg, M, N, total[mt], out_vec_ok);
+      store_out4(out, ldo, row0 + mt * 16 + r16, out_col0 + 4 * kg, M, N, total[mt], out_vec_ok);
   }
 }
 
@@ -869,7 +870,10 @@ static int launch_mid(elem_t* out, const elem_t* act, const elem_t* w, int M, in
     (void)hipFuncSetAttribute((const void*)gemm_mid_kernel<MT, KH, SWIGLU>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     configured = true;
   }
-  gemm_mid_kernel<MT, KH, SWIGLU><<<(N + COLS - 1) / COLS, 512, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok);
+  // Blocks of 16 MT rows side by side: those of a weight tile run at about the same time, and on the same
+  // chip part when the grid's width is a multiple of eight, so that all but one find it in its cache.
+  const dim3 grid((N + COLS - 1) / COLS, (M + 16 * MT - 1) / (16 * MT));
+  gemm_mid_kernel<MT, KH, SWIGLU><<<grid, 512, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok);
   return vk_check_launch("gemm_mid");
 }
 
@@ -890,8 +894,9 @@ extern "C" {
 // kernel: 0 = choose by size, 1 = skinny (M <= 64), 2 = tiled (pipelined if K allows), 3 = tiled through
 // registers, 4..6 = pipelined with 2..4 stages, 7 = skinny with two weight tiles per workgroup where it has
 // such a variant, 8, 9 and 10 = activations shared through LDS with 64, 32 and 128 weight rows per workgroup
-// (17 to 64 rows), 11 = skinny with two activation tiles resident in registers (17 to 32 rows of 16-bit
-// elements, K <= 4096); for measurements and tests.  The result does not depend on the choice.
+// (17 to 512 rows, in blocks of 64 rows), 11 = skinny with two activation tiles resident in registers (17 to
+// 32 rows of 16-bit elements, K <= 4096), 12 = as 9 in blocks of 32 rows; for measurements and tests.  The
+// result does not depend on the choice.
 int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K, int64_t lda, int64_t ldo,
             int kernel, hipStream_t st) {
   VK_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
@@ -900,7 +905,7 @@ int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K
              (long long)lda, VK_VEC);
   VK_REQUIRE(ldo >= N, "gemm: output row stride %lld is smaller than N=%d", (long long)ldo, N);
   VK_REQUIRE(((uintptr_t)act % 16) == 0 && ((uintptr_t)w % 16) == 0, "gemm: operands must be 16-byte aligned");
-  VK_REQUIRE(kernel >= 0 && kernel <= 11, "gemm: unknown kernel %d", kernel);
+  VK_REQUIRE(kernel >= 0 && kernel <= 12, "gemm: unknown kernel %d", kernel);
   if (M == 0) return 0;
   const int vec_ok = (ldo % 4 == 0) && ((uintptr_t)out % 16 == 0);
   // Measured on Qwen3-8B shapes (MI355X).  Up to 16 rows: the streaming kernel.  17 to 32 rows of 16-bit
@@ -920,16 +925,32 @@ int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K
     else if (M <= 64 && K % KC == 0) {
       if (N >= 24576) kernel = 10;
       else if (N >= 8192) kernel = 8;
+      // So few weight rows that workgroups of 32 of them leave half the compute units idle: two blocks
+      // of 32 rows each, side by side (64 rows, 4096 x 12288: 55 -> 45 us).
+      else if (M > 32 && 2 * ((N + 31) / 32) <= device_cus() && (M > 40 || K > SK_WAVES * KC)) kernel = 12;
       else if (M > 40) kernel = 9;
       else if (K <= SK_WAVES * KC || (N + 15) / 16 <= device_cus()) kernel = N >= 6144 ? 7 : 1;
       else kernel = 9;
     }
     else if (M <= 64) kernel = (N >= 16384 && M > 32) ? 2 : (N >= 6144 ? 7 : 1);
+    else if (M <= 256 && K % KC == 0 && N < 16384) {
+      // 65 to 256 rows and few weight rows: the tile kernel would have a workgroup or less per compute
+      // unit, each walking all of K on its own (4096 x 12288 takes it 170 us at any of these sizes); the
+      // kernel above in blocks of 64 rows fills the chip (100 rows: 51 us, 200 rows: 82 us).
+      const int blocks = (M + 63) / 64;
+      if (N >= 8192) kernel = blocks <= 3 ? 8 : 2;
+      else if (blocks == 2) kernel = N <= 4096 ? 9 : 8;
+      else kernel = (K <= SK_WAVES * KC && N >= 6144) ? 2 : 8;
+    }
     else kernel = 2;
   }
+  if (kernel == 12) {      // 32 weight rows per workgroup, four chunks in work, blocks of 32 rows
+    VK_REQUIRE(M > 16 && M <= 512 && K % KC == 0, "gemm: the mid kernel takes 17 to 512 rows and K a multiple of %d", KC);
+    return launch_mid<2, 4>(out, act, w, M, N, K, lda, ldo, vec_ok, st);
+  }
   if (kernel >= 8 && kernel <= 10) {
-    VK_REQUIRE(M > 16 && M <= 64 && K % KC == 0, "gemm: the mid kernel takes 17 to 64 rows and K a multiple of %d", KC);
-    const int mt = (M + 15) / 16;
+    VK_REQUIRE(M > 16 && M <= 512 && K % KC == 0, "gemm: the mid kernel takes 17 to 512 rows and K a multiple of %d", KC);
+    const int mt = M > 64 ? 4 : (M + 15) / 16;       // more than 64 rows: blocks of 64
     if (kernel == 10) {     // 128 weight rows per workgroup, every wave all chunks of its tile
       if (mt == 2) return launch_mid<2, 1>(out, act, w, M, N, K, lda, ldo, vec_ok, st);
       return launch_mid<4, 1>(out, act, w, M, N, K, lda, ldo, vec_ok, st);
