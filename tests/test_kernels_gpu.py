@@ -39,6 +39,8 @@ def test_gemm(dtype, M, N, K):
     ref = (a.double() @ w.double().t()).float()
     got_t = k.gemm(a.cuda(), w.cuda(), kernel=2)
     torch.testing.assert_close(got_t.float().cpu(), ref.to(dtype).float(), **tol(dtype))
+    if K % (64 if dtype == torch.bfloat16 else 32) == 0:
+        assert torch.equal(k.gemm(a.cuda(), w.cuda(), kernel=13), got_t), "64 weight rows per workgroup"
     if 64 < M <= 512 and K % 512 == 0:
         for code in (0, 8, 9, 10, 12):  # blocks of 64 (12: of 32) rows through the kernels that share activations through LDS
             assert torch.equal(k.gemm(a.cuda(), w.cuda(), kernel=code), got_t), code

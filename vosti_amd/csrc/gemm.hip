@@ -514,44 +514,57 @@ __device__ __forceinline__ void wait_vmcnt(int n) {
 // gate, those with wn = 1 the up projection), and at the end the up values pass through LDS to the
 // waves that hold the gate values, which write  silu(g) * u  with g and u rounded to the element type
 // first: the bits of the plain projection followed by swiglu_kernel.
-template <int S, bool WHOLE, bool SWIGLU>
+// 16 bytes per lane from global memory into LDS at dst + 16 * lane.  In a function of its own: called
+// with template-dependent arguments from inside the kernel template, the builtin keeps the compiler
+// from emitting the kernel's host-side stub.
+__device__ __forceinline__ void pipe_load_to_lds16(const elem_t* src, unsigned char* dst) {
+  __builtin_amdgcn_global_load_lds(src, (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+}
+
+// FNW: 16-row weight fragments per wave, 4 (a workgroup takes 128 weight rows) or 2 (64: twice the
+// workgroups, for grids that would leave compute units with one workgroup or none).
+template <int S, bool WHOLE, bool SWIGLU, int FNW = 4>
 __global__ __launch_bounds__(256, 2) void gemm_pipe_kernel(elem_t* __restrict__ out, const elem_t* __restrict__ act,
                                                         const elem_t* __restrict__ w, int M, int N, int K,
                                                         int64_t lda, int64_t ldo, int out_vec_ok) {
-  constexpr int TILE_BYTES = 128 * T_ROWB, STAGE_BYTES = 2 * TILE_BYTES;
+  static_assert(FNW == 4 || (FNW == 2 && !SWIGLU), "two or four weight fragments per wave");
+  constexpr int BN = 32 * FNW;                          // weight rows of the workgroup
+  constexpr int W_BYTES = BN * T_ROWB, STAGE_BYTES = W_BYTES + 128 * T_ROWB;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];   // [stage][w tile, act tile]
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r16 = lane & 15, kg = lane >> 4;
   const int wn = wave & 1, wm = wave >> 1;
-  const int n_blk = blockIdx.x * (SWIGLU ? 64 : 128), m_blk = blockIdx.y * 128;
+  const int n_blk = blockIdx.x * (SWIGLU ? 64 : BN), m_blk = blockIdx.y * 128;
   const int ntiles = K / (2 * VK_SLAB);
 
   // A wave-level load moves 8 rows x 128 bytes; lane i fills LDS slot i of the 1 KB block, which is
   // row i/8, physical 16-byte column i%8, i.e. logical column (i%8) ^ (i/8).
   const int lr = lane >> 3, lc = (lane & 7) ^ lr;
-  const elem_t* gw[4];
+  const elem_t* gw[FNW];
   const elem_t* ga[4];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int row = (wave * 4 + j) * 8 + lr;
+  for (int j = 0; j < FNW; ++j) {
+    const int row = (wave * FNW + j) * 8 + lr;
     const int wrow = SWIGLU ? (row < 64 ? min(n_blk + row, N - 1) : N + min(n_blk + row - 64, N - 1)) : min(n_blk + row, N - 1);
     gw[j] = w + (int64_t)wrow * K + lc * VK_VEC;
-    ga[j] = act + (int64_t)min(m_blk + row, M - 1) * lda + lc * VK_VEC;
   }
-  auto issue = [&](int kt) {
-    unsigned char* base = lds + (kt % S) * STAGE_BYTES + (wave * 4) * 8 * T_ROWB;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) ga[j] = act + (int64_t)min(m_blk + (wave * 4 + j) * 8 + lr, M - 1) * lda + lc * VK_VEC;
+  auto issue = [&](int kt) {                 // FNW + 4 loads per wave
+    unsigned char* base = lds + (kt % S) * STAGE_BYTES;
     const int k = kt * 2 * VK_SLAB;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      __builtin_amdgcn_global_load_lds(gw[j] + k, (__attribute__((address_space(3))) void*)(base + j * 8 * T_ROWB), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds(ga[j] + k, (__attribute__((address_space(3))) void*)(base + TILE_BYTES + j * 8 * T_ROWB), 16, 0, 0);
-    }
+    for (int j = 0; j < FNW; ++j)
+      pipe_load_to_lds16(gw[j] + k, base + (wave * FNW + j) * 8 * T_ROWB);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      pipe_load_to_lds16(ga[j] + k, base + W_BYTES + (wave * 4 + j) * 8 * T_ROWB);
   };
 
-  f32x4 acc[4][4], total[4][4];
+  f32x4 acc[FNW][4], total[FNW][4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < FNW; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -563,41 +576,40 @@ __global__ __launch_bounds__(256, 2) void gemm_pipe_kernel(elem_t* __restrict__ 
     if (p < ntiles) issue(p);
 
   auto step = [&](int kt) {
-    // Tile kt has landed once at most the loads of the tiles after it are outstanding (8 per tile and wave).
+    // Tile kt has landed once at most the loads of the tiles after it are outstanding (FNW + 4 per tile and wave).
     const int later = min(S - 2, ntiles - 1 - kt);
-    wait_vmcnt(8 * later);
+    wait_vmcnt((FNW + 4) * later);
     __syncthreads();       // every wave's part of tile kt is there; everyone is done with tile kt-1's buffer
     if (kt + S - 1 < ntiles) issue(kt + S - 1);
     const unsigned char* base = lds + (kt % S) * STAGE_BYTES;
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
-      frag_t wf[4], af[4];
+      frag_t wf[FNW], af[4];
       const int col = ((s * 4 + kg) ^ (r16 & 7)) * 16;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        wf[i] = *reinterpret_cast<const frag_t*>(base + (wn * 64 + i * 16 + r16) * T_ROWB + col);
-        af[i] = *reinterpret_cast<const frag_t*>(base + TILE_BYTES + (wm * 64 + i * 16 + r16) * T_ROWB + col);
-      }
+      for (int i = 0; i < FNW; ++i) wf[i] = *reinterpret_cast<const frag_t*>(base + (wn * 16 * FNW + i * 16 + r16) * T_ROWB + col);
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < 4; ++i) af[i] = *reinterpret_cast<const frag_t*>(base + W_BYTES + (wm * 64 + i * 16 + r16) * T_ROWB + col);
+#pragma unroll
+      for (int i = 0; i < FNW; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[i][j] = mma_slab(wf[i], af[j], acc[i][j]);
     }
 #ifdef VK_BF16
     // Order for the scheduler: the first slab's reads, then the second slab's reads one by one between
     // the first slab's MFMAs, so that they return while the matrix unit works.
-    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);     // 8 LDS reads
+    __builtin_amdgcn_sched_group_barrier(0x100, FNW + 4, 0);     // the first slab's LDS reads
 #pragma unroll
-    for (int q = 0; q < 8; ++q) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);   // 2 MFMA
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // 1 LDS read
+    for (int q = 0; q < FNW + 4; ++q) {
+      __builtin_amdgcn_sched_group_barrier(0x008, FNW == 4 ? 2 : 1, 0);   // MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                  // 1 LDS read
     }
-    __builtin_amdgcn_sched_group_barrier(0x008, 16, 0);    // the second slab's MFMAs
+    __builtin_amdgcn_sched_group_barrier(0x008, FNW == 4 ? 16 : 10, 0);   // the first slab's other MFMAs and the second slab's
 #endif
   };
   auto close_chunk = [&]() {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < FNW; ++i)
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         total[i][j].x = total[i][j].x + acc[i][j].x;
@@ -622,7 +634,7 @@ __global__ __launch_bounds__(256, 2) void gemm_pipe_kernel(elem_t* __restrict__ 
     }
   }
 
-  if (SWIGLU) {
+  if constexpr (SWIGLU) {
     // The two waves of a row block split the 64 output columns: the gate wave keeps columns 0..31 and
     // gets their up values, the up wave keeps columns 32..63 and gets their gate values.
     __syncthreads();            // the last tile has been read: LDS is free
@@ -654,27 +666,28 @@ __global__ __launch_bounds__(256, 2) void gemm_pipe_kernel(elem_t* __restrict__ 
     return;
   }
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < FNW; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j)
-      store_out4(out, ldo, m_blk + wm * 64 + j * 16 + r16, n_blk + wn * 64 + i * 16 + 4 * kg, M, N, total[i][j],
+      store_out4(out, ldo, m_blk + wm * 64 + j * 16 + r16, n_blk + wn * 16 * FNW + i * 16 + 4 * kg, M, N, total[i][j],
                  out_vec_ok);
 }
 
-template <int S, bool SWIGLU = false>
+template <int S, bool SWIGLU = false, int FNW = 4>
 static int launch_pipe(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K, int64_t lda, int64_t ldo,
                        int vec_ok, hipStream_t st) {
-  const size_t smem = (size_t)S * 2 * 128 * T_ROWB;     // also holds the 32 KB that SWIGLU passes between waves
+  constexpr int BN = SWIGLU ? 64 : 32 * FNW;                         // output columns of a workgroup
+  const size_t smem = (size_t)S * (32 * FNW + 128) * T_ROWB;         // also holds the 32 KB that SWIGLU passes between waves
   static bool configured = false;
   if (!configured) {
-    (void)hipFuncSetAttribute((const void*)gemm_pipe_kernel<S, true, SWIGLU>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    (void)hipFuncSetAttribute((const void*)gemm_pipe_kernel<S, false, SWIGLU>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    (void)hipFuncSetAttribute((const void*)gemm_pipe_kernel<S, true, SWIGLU, FNW>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    (void)hipFuncSetAttribute((const void*)gemm_pipe_kernel<S, false, SWIGLU, FNW>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     configured = true;
   }
-  dim3 grid((N + (SWIGLU ? 63 : 127)) / (SWIGLU ? 64 : 128), (M + 127) / 128);
+  dim3 grid((N + BN - 1) / BN, (M + 127) / 128);
   VK_REQUIRE(grid.y <= 65535, "gemm: too many rows (%d)", M);
-  if (K % KC == 0) gemm_pipe_kernel<S, true, SWIGLU><<<grid, 256, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok);
-  else gemm_pipe_kernel<S, false, SWIGLU><<<grid, 256, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok);
+  if (K % KC == 0) gemm_pipe_kernel<S, true, SWIGLU, FNW><<<grid, 256, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok);
+  else gemm_pipe_kernel<S, false, SWIGLU, FNW><<<grid, 256, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok);
   return vk_check_launch("gemm_pipe");
 }
 
@@ -895,8 +908,8 @@ extern "C" {
 // registers, 4..6 = pipelined with 2..4 stages, 7 = skinny with two weight tiles per workgroup where it has
 // such a variant, 8, 9 and 10 = activations shared through LDS with 64, 32 and 128 weight rows per workgroup
 // (17 to 512 rows, in blocks of 64 rows), 11 = skinny with two activation tiles resident in registers (17 to
-// 32 rows of 16-bit elements, K <= 4096), 12 = as 9 in blocks of 32 rows; for measurements and tests.  The
-// result does not depend on the choice.
+// 32 rows of 16-bit elements, K <= 4096), 12 = as 9 in blocks of 32 rows, 13 = pipelined with 64 weight rows
+// per workgroup; for measurements and tests.  The result does not depend on the choice.
 int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K, int64_t lda, int64_t ldo,
             int kernel, hipStream_t st) {
   VK_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
@@ -905,7 +918,7 @@ int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K
              (long long)lda, VK_VEC);
   VK_REQUIRE(ldo >= N, "gemm: output row stride %lld is smaller than N=%d", (long long)ldo, N);
   VK_REQUIRE(((uintptr_t)act % 16) == 0 && ((uintptr_t)w % 16) == 0, "gemm: operands must be 16-byte aligned");
-  VK_REQUIRE(kernel >= 0 && kernel <= 12, "gemm: unknown kernel %d", kernel);
+  VK_REQUIRE(kernel >= 0 && kernel <= 13, "gemm: unknown kernel %d", kernel);
   if (M == 0) return 0;
   const int vec_ok = (ldo % 4 == 0) && ((uintptr_t)out % 16 == 0);
   // Measured on Qwen3-8B shapes (MI355X).  Up to 16 rows: the streaming kernel.  17 to 32 rows of 16-bit
@@ -1031,7 +1044,14 @@ int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K
   if (kernel == 5 && k_whole) return launch_pipe<3>(out, act, w, M, N, K, lda, ldo, vec_ok, st);
   if (kernel == 6 && k_whole) return launch_pipe<4>(out, act, w, M, N, K, lda, ldo, vec_ok, st);
   // Two stages of 32 KB leave room for two workgroups per compute unit, which hides more latency than a third stage.
-  if (k_whole) return launch_pipe<2>(out, act, w, M, N, K, lda, ldo, vec_ok, st);
+  if (k_whole) {
+    // No more 128 x 128 tiles than compute units: 64 weight rows a workgroup, twice as many of them
+    // (512 rows, 4096 x 12288: 163 -> 145 us; a workgroup alone on its compute unit is bound by what one
+    // compute unit can read, whatever the number of stages).
+    const int64_t tiles = (int64_t)((N + 127) / 128) * ((M + 127) / 128);
+    if (kernel == 13 || (by_size && tiles <= device_cus())) return launch_pipe<2, false, 2>(out, act, w, M, N, K, lda, ldo, vec_ok, st);
+    return launch_pipe<2>(out, act, w, M, N, K, lda, ldo, vec_ok, st);
+  }
   return launch_tiled<4, 4>(out, act, w, M, N, K, lda, ldo, vec_ok, st);
 }
 

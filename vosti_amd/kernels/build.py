@@ -14,6 +14,7 @@ that a long first build is visibly alive.
 """
 from __future__ import annotations
 
+import ctypes
 import hashlib
 import os
 import shutil
@@ -135,6 +136,13 @@ def build(name: str, verbose: bool = True) -> Path:
     if name != "host":
         link.insert(1, f"--offload-arch={GPU_ARCH}")
     _run(link, out.name)
+    # A kernel whose host-side stub the compiler left out shows as an undefined symbol only when the
+    # library is loaded: find out now, not at the first use on a GPU.
+    try:
+        ctypes.CDLL(str(tmp), mode=os.RTLD_NOW)
+    except OSError as e:
+        tmp.unlink(missing_ok=True)
+        raise RuntimeError(f"{out.name} was linked but does not load: {e}") from None
     os.replace(tmp, out)
     Path(str(out) + ".srchash").write_text(source_hash(name) + "\n")
     if verbose:
