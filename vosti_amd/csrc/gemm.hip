@@ -526,7 +526,7 @@ __device__ __forceinline__ void pipe_load_to_lds16(const elem_t* src, unsigned c
 template <int S, bool WHOLE, bool SWIGLU, int FNW = 4>
 __global__ __launch_bounds__(256, 2) void gemm_pipe_kernel(elem_t* __restrict__ out, const elem_t* __restrict__ act,
                                                         const elem_t* __restrict__ w, int M, int N, int K,
-                                                        int64_t lda, int64_t ldo, int out_vec_ok) {
+                                                        int64_t lda, int64_t ldo, int out_vec_ok, int band_w) {
   static_assert(FNW == 4 || (FNW == 2 && !SWIGLU), "two or four weight fragments per wave");
   constexpr int BN = 32 * FNW;                          // weight rows of the workgroup
   constexpr int W_BYTES = BN * T_ROWB, STAGE_BYTES = W_BYTES + 128 * T_ROWB;
@@ -535,7 +535,20 @@ __global__ __launch_bounds__(256, 2) void gemm_pipe_kernel(elem_t* __restrict__ 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r16 = lane & 15, kg = lane >> 4;
   const int wn = wave & 1, wm = wave >> 1;
-  const int n_blk = blockIdx.x * (SWIGLU ? 64 : BN), m_blk = blockIdx.y * 128;
+  // Workgroups start in the order of their linear index.  That order walks bands of band_w column
+  // blocks: all row blocks of a band before the next band, so that a band's weights are read from HBM
+  // once and found in the caches by the other row blocks (a matrix larger than the memory-side cache
+  // would otherwise be streamed once per row block).
+  int nb = blockIdx.x, mb = blockIdx.y;
+  if (band_w < (int)gridDim.x) {
+    const int lin = blockIdx.y * gridDim.x + blockIdx.x;
+    const int per_band = band_w * gridDim.y;
+    const int band = lin / per_band, r = lin - band * per_band;
+    const int w_here = min(band_w, (int)gridDim.x - band * band_w);
+    mb = r / w_here;
+    nb = band * band_w + (r - mb * w_here);
+  }
+  const int n_blk = nb * (SWIGLU ? 64 : BN), m_blk = mb * 128;
   const int ntiles = K / (2 * VK_SLAB);
 
   // A wave-level load moves 8 rows x 128 bytes; lane i fills LDS slot i of the 1 KB block, which is
@@ -673,6 +686,14 @@ __global__ __launch_bounds__(256, 2) void gemm_pipe_kernel(elem_t* __restrict__ 
                  out_vec_ok);
 }
 
+// Column blocks of a band in the tile kernel (0: no bands).  64: the 512 workgroups that run at a time
+// then are 8 row blocks of 64 column blocks, and the 64 of them on a chip part (workgroup i runs on part
+// i % 8) are 8 row blocks of 8 column blocks: the fewest distinct tiles for its cache.  Measured on
+// MI355X, gate/up with SwiGLU at 2,048 to 8,192 rows: 12,288 x 4,096 weights 950 -> 1,090 TFLOP/s,
+// 25,600 x 5,120 (524 MB, more than the memory-side cache holds) 600 -> 1,040; 51 or 76 column blocks,
+// which move a column block from part to part, 780 to 830.
+static int pipe_band_blocks = 64;
+
 template <int S, bool SWIGLU = false, int FNW = 4>
 static int launch_pipe(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K, int64_t lda, int64_t ldo,
                        int vec_ok, hipStream_t st) {
@@ -686,8 +707,9 @@ static int launch_pipe(elem_t* out, const elem_t* act, const elem_t* w, int M, i
   }
   dim3 grid((N + BN - 1) / BN, (M + 127) / 128);
   VK_REQUIRE(grid.y <= 65535, "gemm: too many rows (%d)", M);
-  if (K % KC == 0) gemm_pipe_kernel<S, true, SWIGLU, FNW><<<grid, 256, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok);
-  else gemm_pipe_kernel<S, false, SWIGLU, FNW><<<grid, 256, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok);
+  const int band_w = (pipe_band_blocks > 0 && grid.y > 1 && (int)grid.x > pipe_band_blocks) ? pipe_band_blocks : (int)grid.x;
+  if (K % KC == 0) gemm_pipe_kernel<S, true, SWIGLU, FNW><<<grid, 256, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok, band_w);
+  else gemm_pipe_kernel<S, false, SWIGLU, FNW><<<grid, 256, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok, band_w);
   return vk_check_launch("gemm_pipe");
 }
 
@@ -903,6 +925,9 @@ static int device_cus() {
 }
 
 extern "C" {
+
+// For measurements: the column blocks of a band of the tile kernel (0: no bands).
+void vk_gemm_set_band_blocks(int blocks) { pipe_band_blocks = blocks; }
 
 // kernel: 0 = choose by size, 1 = skinny (M <= 64), 2 = tiled (pipelined if K allows), 3 = tiled through
 // registers, 4..6 = pipelined with 2..4 stages, 7 = skinny with two weight tiles per workgroup where it has
