@@ -32,7 +32,7 @@ def rand(shape, dtype, seed, scale=1.0):
                                    (65, 130, 520), (130, 96, 1032), (300, 520, 2056), (8, 40, 4104),
                                    (8, 4100, 1024), (3, 72, 512), (33, 200, 1536), (64, 4096, 4608), (17, 90, 5120),
                                    (40, 6200, 1024), (64, 6144, 512), (23, 24, 2048), (48, 24700, 512), (20, 24576, 1024), (31, 6200, 4096), (17, 100, 1536), (9, 130, 12288), (16, 72, 8704), (2, 40, 5120), (100, 200, 1024), (65, 4100, 512), (130, 96, 1536),
-                                   (250, 8200, 512), (129, 300, 4608)])
+                                   (250, 8200, 512), (129, 300, 4608), (300, 8400, 128), (700, 9000, 64)])
 def test_gemm(dtype, M, N, K):
     k = kern(dtype)
     a, w = rand((M, K), dtype, 1), rand((N, K), dtype, 2, 0.1)
@@ -533,7 +533,7 @@ def test_attention_refuses_bad_sizes():
 @pytest.mark.parametrize("M,I,K", [(8, 100, 1024), (16, 256, 4096), (1, 33, 512), (5, 48, 96), (20, 64, 1024),
                                    (100, 100, 1024), (300, 256, 2048), (129, 70, 192), (130, 64, 96), (40, 8200, 128),
                                    (8, 100, 5120), (16, 48, 8192), (3, 64, 4608), (32, 4100, 4096), (17, 33, 512),
-                                   (64, 200, 1024), (33, 64, 5120), (48, 8200, 512), (20, 130, 4608)])
+                                   (64, 200, 1024), (33, 64, 5120), (48, 8200, 512), (20, 130, 4608), (200, 4200, 128), (515, 4500, 64)])
 def test_gemm_swiglu_fused_equals_separate(dtype, M, I, K):
     """The gate/up projection with the activation folded in (the streaming kernel for few rows, the
     pipelined tile kernel for many, the kernel that shares activations through LDS between them) gives
