@@ -60,6 +60,23 @@ def test_gemm(dtype, M, N, K):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("N,K", [(4096, 4096), (6144, 1536), (8200, 1024), (24600, 512), (5120, 5120), (300, 8704), (130, 200)])
+def test_gemm_every_row_count(dtype, N, K):
+    """The kernel is chosen by the sizes, with many borders along the row count (16, 32, 40, 64, 128,
+    256, ...): the first M rows of a product are the same bits whatever M is, and so are the fused
+    gate/up rows."""
+    k = kern(dtype)
+    a, w = rand((330, K), dtype, 5).cuda(), rand((N, K), dtype, 6, K ** -0.5).cuda()
+    full = k.gemm(a, w, kernel=2)
+    torch.testing.assert_close(full.float().cpu(), (a.double().cpu() @ w.double().cpu().t()).to(dtype).float(), **tol(dtype))
+    fused = k.gemm_swiglu(a, w) if N % 2 == 0 else None
+    for M in list(range(1, 70)) + [95, 96, 97, 127, 128, 129, 191, 192, 193, 255, 256, 257, 300, 330]:
+        assert torch.equal(k.gemm(a[:M], w), full[:M]), M
+        if fused is not None:
+            assert torch.equal(k.gemm_swiglu(a[:M], w), fused[:M]), M
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_gemm_fused_qkv_equals_three(dtype):
     # The reference holds this bitwise (kernels/tests/runtime/test_qkv_matmul.py:20-34).
     k = kern(dtype)
