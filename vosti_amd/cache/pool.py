@@ -32,6 +32,7 @@ class CachePool:
         if not windows:
             windows = [0]
         has_state = any(isinstance(s, StateSlotSpec) for s in specs)
+        self.has_state = has_state
         groups = [GroupSpec(w, num_pages if w == 0 else (window_pages or num_pages)) for w in windows]
         # A prefix page holds keys only; a mixer with state of its own could not resume from it.
         self.manager = CacheManager(page_size, groups, num_slots, prefix_cache and not has_state)

@@ -26,6 +26,10 @@ from ..kernels.ops import ATTN_ITEM_ROWS, SEGMENT_KEYS
 from ..parts.base import GroupTables, StepContext
 
 WIDTH_BUCKET = 8       # captured block tables grow in steps of this many pages
+# Captured decode steps have one of these numbers of rows; a step with fewer is filled up with rows that
+# read one key of page 0 and write nothing (the reference pads its graphs likewise,
+# python/vosti_kernels/graph_overlay.py:177-389).
+ROW_BUCKETS = (1, 2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64, 96, 128, 192, 256, 384, 512)
 
 
 @dataclass
@@ -103,11 +107,14 @@ class ModelRunner:
         for e in entries:
             self.cache.commit(e.request_id)
 
-    def _layout(self, entries: list[StepEntry], widths: list[int] | None = None) -> _Layout:
-        """The step's host arrays.  ``widths``: block-table width per group (default: what the step needs)."""
+    def _layout(self, entries: list[StepEntry], widths: list[int] | None = None, rows: int | None = None) -> _Layout:
+        """The step's host arrays.  ``widths``: block-table width per group (default: what the step needs).
+        ``rows``: fill up to this many sequences with padding rows of one token: token 0 at position 0,
+        one key (whatever page 0 holds), slot -1 (nothing is stored), logits wanted like the others."""
         cache, spec = self.cache, self.model.spec
-        S = len(entries)
-        q_lens = [len(e.tokens) for e in entries]
+        real = len(entries)
+        S = max(real, rows or 0)
+        q_lens = [len(e.tokens) for e in entries] + [1] * (S - real)
         T = sum(q_lens)
         starts = []
         for e, n in zip(entries, q_lens):
@@ -115,7 +122,8 @@ class ModelRunner:
                 raise RuntimeError(f"request {e.request_id}: the cache holds pages for {cache.pending(e.request_id)} "
                                    f"pending tokens, the step brings {n}")
             starts.append(cache.length(e.request_id))
-        ids = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries])
+        starts += [0] * (S - real)
+        ids = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries] + [np.zeros(S - real, dtype=np.int64)])
         if ids.min() < 0 or ids.max() >= spec.vocab_size:
             raise ValueError(f"token id out of range [0, {spec.vocab_size})")
         k_len = np.asarray([s + n for s, n in zip(starts, q_lens)], dtype=np.int32)
@@ -124,13 +132,14 @@ class ModelRunner:
         positions = np.concatenate([np.arange(s, s + n, dtype=np.int32) for s, n in zip(starts, q_lens)])
         cu_q = np.zeros(S + 1, dtype=np.int32)
         np.cumsum(q_lens, out=cu_q[1:])
-        state_slots = np.asarray([cache.state_slot(e.request_id) for e in entries], dtype=np.int32)
+        state_slots = np.asarray([cache.state_slot(e.request_id) for e in entries] + [0] * (S - real), dtype=np.int32)
         want = []
         for e, base, n in zip(entries, cu_q[:-1], q_lens):
             for w in e.want:
                 if not 0 <= w < n:
                     raise ValueError(f"request {e.request_id}: wanted place {w} is outside its {n} tokens")
                 want.append(int(base) + w)
+        want += [int(cu_q[s]) for s in range(real, S)]
         prefill_items, decode_items = [], []
         for s, n in enumerate(q_lens):
             if n == 1:
@@ -144,7 +153,7 @@ class ModelRunner:
         for g in range(len(self.pool.group_windows)):
             width = widths[g] if widths else self.needed_width(entries, g)
             table = np.zeros((S, width), dtype=np.int32)
-            slots = np.empty(T, dtype=np.int32)
+            slots = np.full(T, -1, dtype=np.int32)
             for s, e in enumerate(entries):
                 cache.block_table_row(e.request_id, g, width, table[s])
                 cache.slots(e.request_id, g, starts[s], q_lens[s], slots[cu_q[s]:cu_q[s + 1]])
@@ -192,7 +201,9 @@ class ModelRunner:
         P = self.pool.page_size
         widths = [-(-self.needed_width(entries, g) // WIDTH_BUCKET) * WIDTH_BUCKET
                   for g in range(len(self.pool.group_windows))]
-        key = (len(entries), tuple(widths))
+        # A mixer with state of its own would have to be told which rows are padding: no padding then.
+        rows = len(entries) if self.pool.has_state else next((b for b in ROW_BUCKETS if b >= len(entries)), len(entries))
+        key = (rows, tuple(widths))
         cap = self._captured.get(key)
         if cap is None and key not in self._seen:
             # First sight of a signature: eagerly, which also warms up every kernel it uses.
@@ -200,12 +211,11 @@ class ModelRunner:
             self.graph_stats["eager"] += 1
             ids, ctx, want = self.build_context(entries)
             return self.model.forward(ids, ctx, self.pool.entries, want)
-        lay = self._layout(entries, widths)
+        lay = self._layout(entries, widths, rows)
         # Launch geometry is frozen in the graph: it must cover every length the tables can hold.
         cover = min(max(widths) * P, self.model.spec.max_positions)
         if cap is None:
-            T, spec = len(entries), self.model.spec
-            self._attn_scratch(self._max_scratch(T, cover))
+            self._attn_scratch(self._max_scratch(rows, cover))
             staging = torch.empty(lay.total, dtype=torch.int32, pin_memory=True)
             meta = torch.zeros(lay.total, dtype=torch.int32, device="cuda")
             lay.pack(staging.numpy())
@@ -225,7 +235,7 @@ class ModelRunner:
         cap.copied.record()
         cap.graph.replay()
         self.graph_stats["replayed"] += 1
-        return cap.logits
+        return cap.logits[:len(entries)]
 
     def _max_scratch(self, tokens: int, cover: int) -> int:
         """Floats of attention scratch that any mixer of the model needs for ``tokens`` decode rows over ``cover`` keys."""
