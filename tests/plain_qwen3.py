@@ -178,13 +178,14 @@ class PlainQwen3:
         down = linear(swiglu(gate_up, dt), w[p + "mlp.down_proj.weight"], dt)
         return down, residual
 
-    def logits(self, ids: list[int]) -> torch.Tensor:
+    def logits(self, ids: list[int], first_position: int = 0) -> torch.Tensor:
         """Logits at every position of one whole sequence: [len(ids), vocab], float32.
         src/exec/dense_swiglu_model.rs:131-1041; a model without layers is
-        lm_head(rms_norm(embed)) (:276-359)."""
+        lm_head(rms_norm(embed)) (:276-359).  ``first_position``: the sequence stands at
+        positions first_position, first_position + 1, ... (for the invariance tests)."""
         w, dt = self.w, self.dtype
         t = torch.tensor(ids, dtype=torch.int64)
-        positions = torch.arange(len(ids))
+        positions = torch.arange(first_position, first_position + len(ids))
         hidden, residual = embedding(t, w["model.embed_tokens.weight"]), None
         for i in range(self.L):
             hidden, residual = self.layer(i, hidden, residual, positions)

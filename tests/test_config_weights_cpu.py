@@ -146,3 +146,44 @@ def test_type_policy():
     assert convert(bf, torch.bfloat16, keep_f32=True).dtype == torch.bfloat16
     assert convert(bf, torch.float32, keep_f32=False).dtype == torch.float32
     assert convert(torch.ones(3, dtype=torch.int64), torch.bfloat16, keep_f32=False).dtype == torch.int32
+
+
+def test_a_tied_head_is_the_embedding_by_name():
+    """Tying lives in the specification: both parameters carry one tensor name, so they get one tensor."""
+    tied, untied = Qwen3Config(**TINY_A).model_spec(), Qwen3Config(**TINY_B).model_spec()
+    assert tied.names["head.weight"] == tied.names["embedding.weight"] == "model.embed_tokens.weight"
+    assert tied.ignored_names == ("lm_head.weight",) and untied.ignored_names == ()
+    assert untied.names["head.weight"] == "lm_head.weight"
+    model = DecoderModel(tied, None)
+    e = model.expected_tensors()["model.embed_tokens.weight"]
+    assert [type(owner).__name__ for owner, _ in e.owners] == ["TokenEmbedding", "LinearHead"]
+    t = {n: torch.zeros(x.spec.shape) for n, x in model.expected_tensors().items()}
+    model.load_tensors(t)
+    assert model.head.weight is model.embedding.weight
+    # Sharers must agree on the shape.
+    from dataclasses import replace
+    from vosti_amd.config import PartSpec
+    bad = replace(tied, head=PartSpec("linear_head", {"vocab_size": 255, "hidden_size": 64}))
+    with pytest.raises(ValueError, match="shared by parameters of different shapes"):
+        DecoderModel(bad, None).expected_tensors()
+
+
+def test_zero_layers_is_a_configuration():
+    # src/exec/dense_swiglu_model.rs:276-359; fixture tests/support/model_families/qwen3.rs:26-36.
+    c = config_from_dict(hf_dict(TINY_A, num_hidden_layers=0))
+    spec = c.model_spec()
+    assert c.num_hidden_layers == 0 and spec.layers == () and spec.schedule == ()
+    assert sorted(expected_tensor_specs(c)) == ["model.embed_tokens.weight", "model.norm.weight"]
+    with pytest.raises(ConfigError, match="num_hidden_layers"):
+        config_from_dict(hf_dict(TINY_A, num_hidden_layers=-1))
+
+
+def test_launcher_families_come_from_the_registry():
+    from vosti_amd.config import register_architecture
+    from vosti_amd.launch import families
+    assert families()["qwen3"] == "Qwen3ForCausalLM"
+
+    @register_architecture("ProbeForCausalLM", model_type="probe_family")
+    class Probe:
+        pass
+    assert families()["probe_family"] == "ProbeForCausalLM"

@@ -18,8 +18,10 @@ def kern(dtype):
 
 
 def tol(dtype):
-    # One rounding to the element type of a value of order 1, plus accumulation differences.
-    return dict(rtol=2e-2, atol=2e-2) if dtype == torch.bfloat16 else dict(rtol=2e-5, atol=2e-5)
+    # bfloat16: the plain function rounds where the kernel does, so the two differ where a sum taken in
+    # another order lands on the neighbouring value: one step of the type (2^-8 to 2^-7 of the value),
+    # and as much of the operands' size where the value is a difference of them.
+    return dict(rtol=2 ** -7, atol=2 ** -8) if dtype == torch.bfloat16 else dict(rtol=2e-5, atol=2e-5)
 
 
 def rand(shape, dtype, seed, scale=1.0):
@@ -296,7 +298,7 @@ def build_cache(kk, vv, P, n_pages, seed, dtype, poison=None):
     return kc, vc, table
 
 
-def run_attention(k, q_list, kk, vv, P, dtype, window=0, poison=None, decode_split=None, seed=0, prompt_mode=0):
+def run_attention(k, q_list, kk, vv, P, dtype, window=0, poison=None, decode_split=None, seed=0, prompt_mode=0, decode_mode=1):
     n_pages = sum(-(-x.shape[0] // P) for x in kk) + 3
     kc, vc, table = build_cache(kk, vv, P, n_pages, seed, dtype, poison)
     q = torch.cat(q_list).cuda()
@@ -314,8 +316,8 @@ def run_attention(k, q_list, kk, vv, P, dtype, window=0, poison=None, decode_spl
     if dec:
         items = torch.tensor(dec, dtype=torch.int32).cuda()
         nseg = -(-int(k_len.max()) // 256) + (1 if decode_split else 0)    # more segments than needed are harmless
-        scratch = torch.full((k.attn_scratch_floats(q.shape[0], q.shape[1], d, nseg),), float("nan"), device="cuda")
-        k.paged_attention(*args, items, mode=1, nseg=nseg, scratch=scratch, **kw)
+        scratch = torch.full((k.attn_scratch_floats(len(dec), q.shape[1], d, nseg),), float("nan"), device="cuda")    # by decoded token, not by row of the step
+        k.paged_attention(*args, items, mode=decode_mode, nseg=nseg, scratch=scratch, **kw)
     return out.cpu()
 
 
@@ -390,15 +392,9 @@ def test_attention_many_decoded_tokens(dtype):
         q_list = [rand((1, nq, d), dtype, 10 + i) for i in range(24)]
         kk = [rand((n, nkv, d), dtype, 40 + i) for i, n in enumerate(lens)]
         vv = [rand((n, nkv, d), dtype, 70 + i) for i, n in enumerate(lens)]
-        try:
-            k.lib.vk_attn_set_decode_variant(2)
-            got = run_attention(k, q_list, kk, vv, P, dtype, window=window, poison=float("nan"))
-            k.lib.vk_attn_set_decode_variant(1)
-            whole = run_attention(k, q_list, kk, vv, P, dtype, window=window, poison=float("nan"), seed=4)
-            k.lib.vk_attn_set_decode_variant(3)
-            by_wave = run_attention(k, q_list, kk, vv, P, dtype, window=window, poison=float("nan"), seed=5)
-        finally:
-            k.lib.vk_attn_set_decode_variant(0)
+        got = run_attention(k, q_list, kk, vv, P, dtype, window=window, poison=float("nan"), decode_mode=4)
+        whole = run_attention(k, q_list, kk, vv, P, dtype, window=window, poison=float("nan"), seed=4, decode_mode=3)
+        by_wave = run_attention(k, q_list, kk, vv, P, dtype, window=window, poison=float("nan"), seed=5, decode_mode=5)
         assert torch.equal(whole, got) and torch.equal(by_wave, got)
         for i in (0, 11, 23):
             ref = plain.attention(q_list[i], kk[i], vv[i], d ** -0.5, dtype, window=window)
@@ -419,13 +415,8 @@ def test_attention_decode_kernels_agree(dtype, nq, nkv, d, P, window):
     q_list = [rand((1, nq, d), dtype, 10 + i) for i in range(len(lens))]
     kk = [rand((n, nkv, d), dtype, 40 + i) for i, n in enumerate(lens)]
     vv = [rand((n, nkv, d), dtype, 70 + i) for i, n in enumerate(lens)]
-    try:
-        k.lib.vk_attn_set_decode_variant(2)
-        got = run_attention(k, q_list, kk, vv, P, dtype, window=window, poison=float("nan"))
-        k.lib.vk_attn_set_decode_variant(3)
-        by_wave = run_attention(k, q_list, kk, vv, P, dtype, window=window, poison=float("nan"), seed=5)
-    finally:
-        k.lib.vk_attn_set_decode_variant(0)
+    got = run_attention(k, q_list, kk, vv, P, dtype, window=window, poison=float("nan"), decode_mode=4)
+    by_wave = run_attention(k, q_list, kk, vv, P, dtype, window=window, poison=float("nan"), seed=5, decode_mode=5)
     assert torch.equal(by_wave, got)
     for i in range(len(lens)):
         ref = plain.attention(q_list[i], kk[i], vv[i], d ** -0.5, dtype, window=window)
@@ -559,5 +550,46 @@ def test_gemm_swiglu_fused_equals_separate(dtype, M, I, K):
     k = kern(dtype)
     a, w = rand((M, K), dtype, 1).cuda(), rand((2 * I, K), dtype, 2, K ** -0.5).cuda()    # projections of order 1
     got = k.gemm_swiglu(a, w)
-    assert torch.equal(got, k.swiglu(k.gemm(a, w, kernel=2)))
-    torch.testing.assert_close(got.float().cpu(), plain.swiglu(plain.linear(a.cpu(), w.cpu(), dtype), dtype), **tol(dtype))
+    gu = k.gemm(a, w, kernel=2)
+    assert torch.equal(got, k.swiglu(gu))
+    # Each of the two roundings against its plain function on the same input: the projection, then the
+    # activation of the projection's own output (a flip of the first carried through the second is
+    # several steps of the type).
+    torch.testing.assert_close(gu.float().cpu(), plain.linear(a.cpu(), w.cpu(), dtype), **tol(dtype))
+    torch.testing.assert_close(got.float().cpu(), plain.swiglu(gu.cpu(), dtype), **tol(dtype))
+
+
+def test_attention_rounds_probabilities_as_the_reference_does():
+    """bfloat16: P is rounded to the element type for P.V while the normaliser sums the unrounded P
+    (kernels/triton_kernels/fattn_paged.py:236-244).  On inputs where the rounding errors add up the
+    kernels agree with that and with neither of the two other ways of rounding, for prompt rows and
+    for decoded rows."""
+    from test_plain_cpu import attention_variant, rounding_probe
+    dtype = torch.bfloat16
+    k = kern(dtype)
+    q, kk, v = rounding_probe()
+    T, d = q.shape
+    q3, k3, v3 = (t.to(dtype)[:, None, :] for t in (q, kk, v))
+    frac = lambda a, b: (a != b).float().mean().item()
+    variants = {how: attention_variant(q, kk, v, 1.0, how) for how in ("reference", "unrounded", "both")}
+
+    def run(q_rows, q_list_k):
+        n_pages = 4
+        kc, vc, table = build_cache([k3], [v3], 16, n_pages, 0, dtype, None)
+        out = torch.zeros(len(q_rows), 1, d, dtype=dtype, device="cuda")
+        cu = torch.tensor([0, len(q_rows)], dtype=torch.int32).cuda()
+        klen = torch.tensor([q_list_k], dtype=torch.int32).cuda()
+        args = (q3[q_rows].contiguous().cuda(), kc.cuda(), vc.cuda(), table.cuda(), cu, klen)
+        if len(q_rows) > 1:
+            k.paged_attention(*args, torch.tensor([[0, 0]], dtype=torch.int32).cuda(), mode=0, scale=1.0, max_k_len=q_list_k, out=out)
+        else:
+            scratch = torch.empty(k.attn_scratch_floats(1, 1, d, 1), device="cuda")
+            k.paged_attention(*args, torch.tensor([[0, 0]], dtype=torch.int32).cuda(), mode=1, scale=1.0, max_k_len=q_list_k,
+                              nseg=1, scratch=scratch, out=out)
+        return out[:, 0].float().cpu()
+
+    prompt_rows = run(list(range(T)), T)
+    decoded = torch.cat([run([r], r + 1) for r in range(1, T)])
+    for got, sl in ((prompt_rows, slice(0, T)), (decoded, slice(1, T))):
+        assert frac(got, variants["reference"][sl]) < 0.01
+        assert frac(got, variants["unrounded"][sl]) > 0.2 and frac(got, variants["both"][sl]) > 0.2

@@ -4,14 +4,14 @@ import torch
 
 import plain_qwen3 as plain
 from vosti_amd.config import PartSpec
-from vosti_amd.kernels.ops import ATTN_ITEM_ROWS
 
 pytestmark = pytest.mark.gpu
 DTYPES = [torch.float32, torch.bfloat16]
 
 
 def tol(dtype):
-    return dict(rtol=2e-2, atol=2e-2) if dtype == torch.bfloat16 else dict(rtol=2e-5, atol=2e-5)
+    # bfloat16: one step of the type where a sum in another order lands on the neighbouring value.
+    return dict(rtol=2 ** -7, atol=2 ** -8) if dtype == torch.bfloat16 else dict(rtol=2e-5, atol=2e-5)
 
 
 def rand(shape, dtype, seed, scale=1.0):
@@ -39,7 +39,8 @@ def load(part, dtype, seed=0, scale=0.1):
 
 def step_context(kernels, starts, q_lens, page, pages_of, n_pages, window=0):
     """A StepContext for sequences whose logical pages are pages_of[s]."""
-    from vosti_amd.parts import GroupTables, StepContext
+    from vosti_amd.parts import GroupTables, HostStep, StepContext
+    from vosti_amd.parts.standard import Attention
     i32 = lambda v: torch.tensor(v, dtype=torch.int32, device="cuda")
     positions = [p for s, n in zip(starts, q_lens) for p in range(s, s + n)]
     slots = [pages_of[i][p // page] * page + p % page for i, (s, n) in enumerate(zip(starts, q_lens)) for p in range(s, s + n)]
@@ -49,15 +50,15 @@ def step_context(kernels, starts, q_lens, page, pages_of, n_pages, window=0):
     for n in q_lens:
         cu.append(cu[-1] + n)
     k_len = [s + n for s, n in zip(starts, q_lens)]
-    pre = [(i, o) for i, n in enumerate(q_lens) if n > 1 for o in range(0, n, ATTN_ITEM_ROWS)]
-    dec = [(i, 0) for i, n in enumerate(q_lens) if n == 1]
+    host = HostStep(q_lens=list(q_lens), starts=list(starts), k_lens=k_len, state_slots=list(range(len(q_lens))),
+                    k_len_bound=max(k_len))
+    # The arrays the attention part asks of a step, uploaded as the step function would.
+    inputs = {name: i32(arr.tolist()).view(-1, 2) for name, arr in Attention._items_arrays(host).items()}
     scratch = torch.empty(1 << 20, device="cuda")
     return StepContext(kernels=kernels, num_tokens=sum(q_lens), num_seqs=len(q_lens), positions=i32(positions), cu_q=i32(cu),
                        k_len=i32(k_len), state_slots=i32(list(range(len(q_lens)))),
-                       groups=[GroupTables(i32(slots), i32(table), window)],
-                       prefill_items=i32(pre).view(-1, 2), decode_items=i32(dec).view(-1, 2), max_k_len=max(k_len),
-                       max_decode_k_len=max([k for k, n in zip(k_len, q_lens) if n == 1], default=0),
-                       host_q_lens=q_lens, host_starts=starts, attn_scratch=lambda n: scratch)
+                       groups=[GroupTables(i32(slots), i32(table), window)], host=host, inputs=inputs,
+                       workspace=lambda n: scratch)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -80,7 +81,8 @@ def test_embedding_norm_head_swiglu(dtype):
     head = build("head", "linear_head", dtype, vocab_size=77, hidden_size=40, tied=False)
     w = load(head, dtype)
     torch.testing.assert_close(head.forward(x.cuda()).float().cpu(), plain.linear(x, w["weight"], dtype), **tol(dtype))
-    assert build("head", "linear_head", dtype, vocab_size=77, hidden_size=40, tied=True).params() == {}
+    # A tied head is the same part: the architecture names its weight like the embedding's table.
+    assert list(build("head", "linear_head", dtype, vocab_size=77, hidden_size=40, tied=True).params()) == ["weight"]
 
     ffn = build("feed_forward", "swiglu", dtype, hidden_size=40, intermediate_size=56)
     w = load(ffn, dtype)

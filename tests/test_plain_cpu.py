@@ -193,3 +193,93 @@ def test_bfloat16_mode_rounds_where_the_reference_stores(tiny_dirs):
     assert torch.equal(b, b.bfloat16().float())            # logits leave the model in the model type
     err = (a - b).abs().max().item()
     assert 1e-4 < err < 0.1
+
+
+def test_head_norm_comes_before_the_rotation(tiny_dirs):
+    """The q/k head norm is applied before the rotary encoding (src/exec/dense_swiglu_decoder.rs:207-246).
+    What fixes the order beside that text: with the norm first, the vectors that are rotated do not
+    depend on the position, so scores depend on distances only and the logits of a sequence do not
+    change when all its positions are shifted.  With the rotation first, the norm's weights (which
+    differ between the two halves of a rotated pair) scale the pair's two members differently after
+    the rotation, and the invariance is lost.  The swapped model, written out here, fails it."""
+    m = plain.PlainQwen3(tiny_dirs["B"], F32)
+    ids = [11, 400, 7, 7, 250, 33, 1, 499, 60, 61, 62, 5]
+    base = m.logits(ids)
+    for shift in (1, 37, 200):
+        torch.testing.assert_close(m.logits(ids, first_position=shift), base, rtol=1e-4, atol=2e-5)
+
+    class Swapped(plain.PlainQwen3):
+        def layer(self, i, hidden, residual, positions):
+            real_norm, real_rope = plain.head_rms_norm, plain.apply_rope
+            pending = {}
+
+            def norm_later(x, w, eps, dt):      # remember the weight, leave x alone until after the rotation
+                pending[x.shape[1]] = (w, eps)
+                return x
+
+            def rope_then_norm(x, cos, sin, pos, dt):
+                w, eps = pending[x.shape[1]]
+                return real_norm(real_rope(x, cos, sin, pos, dt), w, eps, dt)
+            plain.head_rms_norm, plain.apply_rope = norm_later, rope_then_norm
+            try:
+                return super().layer(i, hidden, residual, positions)
+            finally:
+                plain.head_rms_norm, plain.apply_rope = real_norm, real_rope
+
+    sw = Swapped(tiny_dirs["B"], F32)
+    assert (sw.logits(ids) - base).abs().max() > 1e-3                                  # it is another model
+    assert (sw.logits(ids, first_position=37) - sw.logits(ids)).abs().max() > 1e-3      # and not shift-invariant
+
+
+def attention_variant(q, k, v, scale, how):
+    """One head, all rows, vectorised, with the probabilities' rounding written out three ways:
+    'reference': P rounded to bfloat16 for the product, normaliser from the unrounded P
+    (kernels/triton_kernels/fattn_paged.py:236-244); 'unrounded': nothing rounded; 'both': the
+    normaliser from the rounded P too."""
+    T = q.shape[0]
+    s = (q @ k.t()) * scale
+    s = s.masked_fill(~torch.ones(T, T).tril().bool(), float("-inf"))
+    e = torch.exp(s - s.max(-1, keepdim=True).values)
+    eb = e.bfloat16().float()
+    num = (e if how == "unrounded" else eb) @ v
+    den = (eb if how == "both" else e).sum(-1, keepdim=True)
+    return (num / den).bfloat16().float()
+
+
+def rounding_probe(T=48, d=32, delta=1.046875, seed=23):
+    """Inputs on which the rounding of the probabilities shows: row r sees key 0 with score 0 and keys
+    1..r with score -delta each (scale 1), so every probability but one is exp(-delta) = 0.35103, which
+    bfloat16 rounds up by 0.15 %; the values are positive, so the errors add up instead of cancelling.
+    All inputs are exact in bfloat16."""
+    q = torch.zeros(T, d)
+    q[:, 0] = 1.0
+    k = torch.zeros(T, d)
+    k[1:, 0] = -delta
+    v = (torch.rand(T, d, generator=torch.Generator().manual_seed(seed)) + 0.5).bfloat16().float()
+    return q, k, v
+
+
+def test_probabilities_are_rounded_before_they_meet_the_values():
+    """fattn_paged.py:236-244: p is cast to the value type for the dot product, l_i sums the float32 p.
+    On inputs where the rounding errors add up, the three ways of rounding give visibly different
+    outputs, and the plain attention is the first."""
+    q, k, v = rounding_probe()
+    got = plain.attention(q[:, None], k[:, None], v[:, None], 1.0, torch.bfloat16)[:, 0]
+    frac = lambda a, b: (a != b).float().mean().item()
+    assert frac(got, attention_variant(q, k, v, 1.0, "reference")) < 0.01        # the same but for a summation order
+    assert frac(got, attention_variant(q, k, v, 1.0, "unrounded")) > 0.2
+    assert frac(got, attention_variant(q, k, v, 1.0, "both")) > 0.2
+
+
+def test_a_model_without_layers_is_head_of_norm_of_embedding(tmp_path):
+    # src/exec/dense_swiglu_model.rs:276-359; the reference's fixture is tests/support/model_families/qwen3.rs:26-36.
+    from vosti_amd.config import Qwen3Config
+    from vosti_amd.weights import write_random_model
+    cfg = Qwen3Config(**dict(TINY["A"][0], num_hidden_layers=0, tie_word_embeddings=False))
+    write_random_model(cfg, 4, tmp_path, dtype=torch.float32)
+    m = plain.PlainQwen3(tmp_path, F32)
+    ids = [3, 200, 3, 77]
+    e = m.w["model.embed_tokens.weight"][torch.tensor(ids)]
+    ref = plain.rms_norm(e, m.w["model.norm.weight"], m.eps, F32) @ m.w["lm_head.weight"].t()
+    torch.testing.assert_close(m.logits(ids), ref)
+    assert torch.equal(m.logits(ids)[0], m.logits(ids)[2])       # no layer mixes positions

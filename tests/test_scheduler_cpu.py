@@ -91,7 +91,10 @@ def test_admission_status():
     assert s.add_request(3, [1], 0) == "ZeroMaxTokens"
     assert s.add_request(4, [1], 1, eos_token_ids=(1, 2, 3, 4)) == "TooManyEosTokenIds"
     assert s.add_request(5, [1] * 10, 7) == "HistoryCapacityOverflow"
-    s.plan(); s.commit([5])
+    # src/exec/engine.rs:2718-2720: end tokens that count need at least one id.
+    assert s.add_request(6, [1], 1, eos_token_ids=(), ignore_eos=False) == "EmptyEosTokenIds"
+    assert s.add_request(6, [1], 1, eos_token_ids=(), ignore_eos=True) == "Accepted"
+    s.plan(); s.commit([5, 5])
     assert s.add_request(1, [1], 1) == "DuplicateRequestId"      # ids are never reused
 
 
@@ -274,3 +277,31 @@ def test_outputs_do_not_depend_on_the_schedule(seed):
         assert step < 5000
     assert outputs == want
     assert cache.num_requests() == 0 and cache.available_pages(0) == cache.groups[0].num_pages
+
+
+def test_a_step_that_did_not_run_is_planned_again():
+    """plan, give up, plan: the same rows, nothing lost, and the outputs of the whole run unchanged."""
+    from vosti_amd.engine.scheduler import SchedulerError
+    cache, s = make(pages=12, page=4, seqs=3, budget=8)
+    hist = {0: list(range(10)), 1: [7, 7, 7], 2: list(range(20, 26))}
+    for rid, p in hist.items():
+        s.add_request(rid, list(p), 5)
+    key = lambda rows: [(r.request_id, r.start, tuple(r.tokens), r.sample, r.state_slot, r.output_index) for r in rows]
+    first = s.plan()
+    assert first and cache.pending(first[0].request_id) == len(first[0].tokens)
+    with pytest.raises(SchedulerError, match="before the step planned last"):
+        s.plan()
+    with pytest.raises(SchedulerError, match="nothing was committed"):
+        s.commit([1] * (sum(r.sample for r in first) + 1))
+    s.abort_step()
+    assert all(cache.pending(r.request_id) == 0 for r in first) and cache.check() == ""
+    again = s.plan()
+    assert key(again) == key(first)
+    s.abort_step()
+    # Given up twice, then run to the end: what comes out is what an undisturbed run gives.
+    outs, _ = drive(s, cache, hist)
+    assert outs == {0: expected(range(10), 5), 1: expected([7, 7, 7], 5), 2: expected(range(20, 26), 5)}
+    assert cache.num_requests() == 0 and cache.check() == ""
+    # Giving up when nothing is planned is harmless.
+    s.abort_step()
+    assert s.plan() == []

@@ -6,7 +6,7 @@ from ctypes import POINTER, c_char_p, c_int, c_int32, c_int64, c_uint64, c_void_
 
 from ..kernels import build
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 _LIB = None
 
 
@@ -50,6 +50,8 @@ def host_lib():
     sig("vh_sched_get_plan", None, P, c_void_p, c_void_p)
     sig("vh_sched_commit", I, P, PI, I)
     sig("vh_sched_get_emitted", None, P, c_void_p)
+    sig("vh_sched_abort_step", None, P)
+    sig("vh_sched_num_planned_samples", I, P)
     sig("vh_sched_abort", I, P, U)
     sig("vh_sched_num_waiting", I, P)
     sig("vh_sched_num_running", I, P)

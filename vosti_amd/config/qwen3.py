@@ -100,7 +100,10 @@ class Qwen3Config:
         tie = _get(raw, "tie_word_embeddings", False)
         if not isinstance(tie, bool):
             raise ConfigError("config.json: 'tie_word_embeddings' must be true or false")
-        layers = _pos_int(raw, "num_hidden_layers")
+        # A model without layers is lm_head(rms_norm(embed)) (src/exec/dense_swiglu_model.rs:276-359).
+        layers = _get(raw, "num_hidden_layers")
+        if isinstance(layers, bool) or not isinstance(layers, int) or layers < 0:
+            raise ConfigError(f"config.json: 'num_hidden_layers' must be an integer, zero or more, got {layers!r}")
         if layer_types is not None and len(layer_types) != layers:
             raise ConfigError("config.json: 'layer_types' must have one entry per layer")
         return cls(
@@ -171,8 +174,11 @@ class Qwen3Config:
             final_norm=norm,
             head=PartSpec("linear_head", {"vocab_size": self.vocab_size, "hidden_size": self.hidden_size,
                                           "tied": self.tie_word_embeddings}),
+            # A tied head is the embedding table itself (python/vosti_kernels/model_families/qwen3/physical.py:131-134);
+            # a checkpoint that stores an lm_head.weight beside it is tolerated.
             names={"embedding.weight": "model.embed_tokens.weight", "final_norm.weight": "model.norm.weight",
-                   "head.weight": "lm_head.weight"},
+                   "head.weight": "model.embed_tokens.weight" if self.tie_word_embeddings else "lm_head.weight"},
+            ignored_names=("lm_head.weight",) if self.tie_word_embeddings else (),
         )
         spec.validate()
         return spec

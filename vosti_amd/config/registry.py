@@ -37,6 +37,11 @@ def architecture_names() -> list[str]:
     return sorted(_ARCHITECTURES)
 
 
+def model_types() -> dict[str, str]:
+    """config.json ``model_type`` -> architecture name, for every architecture registered with one."""
+    return dict(_MODEL_TYPES)
+
+
 def resolve_architecture(raw: Mapping[str, Any]) -> str:
     archs = raw.get("architectures")
     if isinstance(archs, (list, tuple)) and archs:

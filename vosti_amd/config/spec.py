@@ -54,7 +54,11 @@ class ModelSpec:
     schedule: tuple[ScheduleEntry, ...]
     final_norm: PartSpec
     head: PartSpec
-    names: Mapping[str, str]    # "embedding.weight", "final_norm.weight", "head.weight" -> tensor names
+    # "embedding.weight", "final_norm.weight", "head.weight" -> tensor names.  Two parameters with the
+    # same tensor name are one tensor: a head tied to the embedding is written so.
+    names: Mapping[str, str]
+    # Tensors that a checkpoint may hold although the model does not use them.
+    ignored_names: tuple[str, ...] = ()
 
     def validate(self) -> None:
         for i, e in enumerate(self.schedule):

@@ -59,8 +59,8 @@ struct AttnArgs {
   const int32_t* cu_q;    // [S + 1]
   const int32_t* k_len;   // [S]
   const int32_t* items;   // [n_items, 2]: (sequence, first row of the item within the step's rows of it)
-  float* part_ml;         // decode: [T * nq * nseg, 2]
-  float* part_acc;        // decode: [T * nq * nseg, d]
+  float* part_ml;         // decode: [n_items * nq * nseg, 2], indexed by the item, not by the token
+  float* part_acc;        // decode: [n_items * nq * nseg, d]
   int bt_stride, nq, nkv, d, P, window, nseg;
   float scale_log2;
 };
@@ -694,7 +694,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
       M = Mn;
     }
   }
-  const int64_t prow = ((int64_t)tok * a.nq + (kvh * G + ht * 16 + row)) * a.nseg + seg;
+  const int64_t prow = ((int64_t)blockIdx.x * a.nq + (kvh * G + ht * 16 + row)) * a.nseg + seg;
   if (cg == 0) {
     a.part_ml[2 * prow] = M;
     a.part_ml[2 * prow + 1] = L;
@@ -794,7 +794,7 @@ __global__ __launch_bounds__(64 * SEG_WAVES, 2) void attn_decode_seg_kernel(Attn
   for (int t = t0; t < t1; ++t) tile(t, true);
   tile(t1, false);
   if (!c.row_ok) return;
-  const int64_t prow = ((int64_t)tok * a.nq + head) * a.nseg + seg;
+  const int64_t prow = ((int64_t)blockIdx.x * a.nq + head) * a.nseg + seg;
   if (c.g == 0) {
     a.part_ml[2 * prow] = M;
     a.part_ml[2 * prow + 1] = L;
@@ -912,7 +912,7 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(AttnArgs a) {
   const int d = a.d;
   float M = -INFINITY, L = 0.f;
   float ACC[4] = {0.f, 0.f, 0.f, 0.f};   // d <= 256
-  const int64_t row0 = ((int64_t)tok * a.nq + head) * a.nseg;
+  const int64_t row0 = ((int64_t)blockIdx.x * a.nq + head) * a.nseg;
   // Four segments are fetched together, then folded one after the other.
   for (int seg0 = seg_begin; seg0 < seg_end; seg0 += 4) {
     float m[4], l[4], v[4][4];
@@ -955,9 +955,10 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(AttnArgs a) {
 
 extern "C" {
 
-// Number of floats of scratch a decode launch needs for `tokens` rows.
-int64_t vk_attn_scratch_floats(int tokens, int nq, int d, int nseg) {
-  const int64_t rows = (int64_t)tokens * nq * nseg;
+// Number of floats of scratch a decode launch needs for `items` decoded tokens (mode 1 items; the
+// prompt rows of the same step need none).
+int64_t vk_attn_scratch_floats(int items, int nq, int d, int nseg) {
+  const int64_t rows = (int64_t)items * nq * nseg;
   return ((rows * 2 + 3) & ~(int64_t)3) + rows * d;
 }
 
@@ -965,14 +966,6 @@ int vk_attn_segment_keys(void) { return TILE_KEYS * SEG_TILES; }
 
 int vk_attn_item_rows(void) { return ITEM_ROWS; }
 
-// For measurements: 0 is the default shape of the workgroups of the prompt kernel, 14 is the other
-// (row tiles per wave * 10 + waves).  The result is the same bits.
-static int vk_prefill_variant = 0;
-void vk_attn_set_prefill_variant(int v) { vk_prefill_variant = v; }
-// 0: the decode kernel is chosen by size, 1: one workgroup per token and kv head where LDS allows,
-// 2: always the split over segments.  The result is the same bits.
-static int vk_decode_variant = 0;
-void vk_attn_set_decode_variant(int v) { vk_decode_variant = v; }
 static int vk_dpad(int d) { return d <= 64 ? 64 : (d <= 128 ? 128 : 256); }
 
 // 1 if prompt rows of this shape go through the kernel that shares key tiles in LDS.
@@ -980,13 +973,16 @@ int vk_attn_prefill_shares_tiles(int d, int P) {
   return (d == 64 || d == 128 || d == 256) && P >= TILE_KEYS && 4 * TILE_KEYS * d * (int)sizeof(elem_t) <= 128 * 1024;
 }
 
-// items: n_items pairs (sequence, first row).  mode 0 and 2: each item is up to
-// vk_attn_item_rows() consecutive rows of the sequence's q_len new tokens
-// (mode 2 forces the kernel that takes every shape; the result is the same).
-// mode 1: each item is one token; the keys are split by segment over nseg
-// workgroups (nseg must cover the longest sequence; scratch must hold
-// vk_attn_scratch_floats(T, ...)) and folded by a second kernel.  The result
-// is the same in all modes.
+// items: n_items pairs (sequence, first row).
+// mode 0: each item is up to vk_attn_item_rows() consecutive rows of the sequence's q_len new tokens;
+//   the kernel is chosen by shape.  mode 2: the same through the kernel that takes every shape,
+//   mode 6: through the one that shares tiles in LDS with four waves instead of eight (tests and
+//   measurements; the result is the same bits).
+// mode 1: each item is one token; the keys are split by segment over nseg workgroups (nseg must cover
+//   the longest sequence; scratch must hold vk_attn_scratch_floats(n_items, ...)) and folded by a
+//   second kernel; the kernel is chosen by shape.  modes 3, 4, 5: the same through a named kernel
+//   (3: all keys of a token in one workgroup where LDS allows, 4: a wave per tile, 5: a wave per
+//   segment; tests and measurements; the same bits).
 int vk_paged_attention(elem_t* out, const elem_t* q, const elem_t* kc, const elem_t* vc,
                        const int32_t* block_table, int bt_stride, const int32_t* cu_q, const int32_t* k_len,
                        const int32_t* items, int n_items, int mode, int nseg, float* scratch, int total_tokens,
@@ -996,7 +992,11 @@ int vk_paged_attention(elem_t* out, const elem_t* q, const elem_t* kc, const ele
   VK_REQUIRE(P >= 8 && (P & (P - 1)) == 0, "attention: page size %d must be a power of two >= 8", P);
   VK_REQUIRE(window >= 0, "attention: window %d must not be negative", window);
   VK_REQUIRE(scale > 0.f, "attention: the score scale must be positive");
-  VK_REQUIRE(mode >= 0 && mode <= 2, "attention: unknown mode %d", mode);
+  VK_REQUIRE(mode >= 0 && mode <= 6, "attention: unknown mode %d", mode);
+  const int vk_prefill_variant = mode == 6 ? 14 : 0;
+  const int vk_decode_variant = mode == 3 ? 1 : (mode == 4 ? 2 : (mode == 5 ? 3 : 0));
+  if (mode == 6) mode = 0;
+  if (mode >= 3) mode = 1;
   if (n_items <= 0) return 0;
   AttnArgs a;
   a.q = q; a.out = out; a.kc = kc; a.vc = vc; a.block_table = block_table; a.cu_q = cu_q; a.k_len = k_len;
@@ -1074,7 +1074,7 @@ int vk_paged_attention(elem_t* out, const elem_t* q, const elem_t* kc, const ele
     }
   }
   a.part_ml = scratch;
-  a.part_acc = scratch + (((int64_t)total_tokens * nq * nseg * 2 + 3) & ~(int64_t)3);
+  a.part_acc = scratch + (((int64_t)n_items * nq * nseg * 2 + 3) & ~(int64_t)3);
   const dim3 grid(n_items, nkv * ((G + 15) / 16), nseg);
   VK_REQUIRE(grid.y <= 65535 && nq <= 65535, "attention: too many heads");
   // Measured on MI355X, bfloat16, head size 128: from one token of 300 keys (15.5 against 17.2 us)

@@ -692,7 +692,7 @@ __global__ __launch_bounds__(256, 2) void gemm_pipe_kernel(elem_t* __restrict__ 
 // MI355X, gate/up with SwiGLU at 2,048 to 8,192 rows: 12,288 x 4,096 weights 950 -> 1,090 TFLOP/s,
 // 25,600 x 5,120 (524 MB, more than the memory-side cache holds) 600 -> 1,040; 51 or 76 column blocks,
 // which move a column block from part to part, 780 to 830.
-static int pipe_band_blocks = 64;
+static const int pipe_band_blocks = 64;
 
 template <int S, bool SWIGLU = false, int FNW = 4>
 static int launch_pipe(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K, int64_t lda, int64_t ldo,
@@ -925,9 +925,6 @@ static int device_cus() {
 }
 
 extern "C" {
-
-// For measurements: the column blocks of a band of the tile kernel (0: no bands).
-void vk_gemm_set_band_blocks(int blocks) { pipe_band_blocks = blocks; }
 
 // kernel: 0 = choose by size, 1 = skinny (M <= 64), 2 = tiled (pipelined if K allows), 3 = tiled through
 // registers, 4..6 = pipelined with 2..4 stages, 7 = skinny with two weight tiles per workgroup where it has

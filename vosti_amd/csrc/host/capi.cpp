@@ -20,7 +20,7 @@ struct SchedulerHandle {
 
 extern "C" {
 
-int vh_abi_version(void) { return 4; }
+int vh_abi_version(void) { return 5; }
 
 // ------------------------------------------------------------ cache manager
 void* vh_cache_create(int page_size, int n_groups, const int* windows, const int* num_pages, int num_slots,
@@ -103,10 +103,14 @@ void vh_sched_get_plan(void* h, int64_t* rows_out, int32_t* tokens_out) {
   }
   if (!SH->tokens.empty()) std::memcpy(tokens_out, SH->tokens.data(), SH->tokens.size() * sizeof(int32_t));
 }
+// Returns the number of emitted tokens, or -1 (nothing committed) if n_sampled is not the number of
+// sampled rows of the plan.
 int vh_sched_commit(void* h, const int32_t* sampled, int n_sampled) {
-  SH->sched.commit(sampled, n_sampled, SH->emitted);
+  if (!SH->sched.commit(sampled, n_sampled, SH->emitted)) return -1;
   return (int)SH->emitted.size();
 }
+void vh_sched_abort_step(void* h) { SH->sched.abort_step(); }
+int vh_sched_num_planned_samples(void* h) { return SH->sched.num_planned_samples(); }
 // out: n x 3 int64 (id, token, finished).
 void vh_sched_get_emitted(void* h, int64_t* out) {
   for (size_t i = 0; i < SH->emitted.size(); ++i) {

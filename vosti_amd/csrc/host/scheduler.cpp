@@ -10,6 +10,7 @@ AdmissionStatus Scheduler::add_request(RequestId id, const int32_t* prompt, int 
                                        const int32_t* eos, int n_eos, bool ignore_eos) {
   if (accepted_.count(id)) return DUPLICATE_REQUEST_ID;
   if (n_prompt <= 0 || prompt == nullptr) return EMPTY_PROMPT;
+  if (n_eos == 0 && !ignore_eos) return EMPTY_EOS_TOKEN_IDS;
   if (n_eos > 3 || n_eos < 0) return TOO_MANY_EOS_TOKEN_IDS;
   if (max_tokens <= 0) return ZERO_MAX_TOKENS;
   if ((int64_t)n_prompt + max_tokens > config_.max_model_len) return HISTORY_CAPACITY_OVERFLOW;
@@ -46,7 +47,7 @@ int Scheduler::page_debt() const {
   return debt;
 }
 
-bool Scheduler::try_rows(std::vector<PlanRow>& rows, std::vector<int32_t>& tokens) {
+int Scheduler::try_rows(std::vector<PlanRow>& rows, std::vector<int32_t>& tokens) {
   rows.clear();
   tokens.clear();
   int used = 0;
@@ -58,7 +59,14 @@ bool Scheduler::try_rows(std::vector<PlanRow>& rows, std::vector<int32_t>& token
     const int remaining = (int)r.tokens.size() - computed;
     const int n = remaining == 1 ? 1 : chunk_for(remaining, budget - used, rows.empty());
     if (n <= 0) continue;
-    if (cache_->extend(id, r.tokens.data() + computed, n) != OK) continue;
+    const Status st = cache_->extend(id, r.tokens.data() + computed, n);
+    if (st == NO_PAGES) continue;            // left out of this step; the others go on
+    if (st != OK) {                          // a step still pending, an unknown request: not a matter of pages
+      for (const PlanRow& done : rows) cache_->abort_step(done.id);
+      rows.clear();
+      tokens.clear();
+      return -1;
+    }
     rows.push_back(PlanRow{id, computed, n, computed + n == (int)r.tokens.size() ? 1 : 0, cache_->state_slot(id),
                            r.generated});
     tokens.insert(tokens.end(), r.tokens.begin() + computed, r.tokens.begin() + computed + n);
@@ -93,18 +101,24 @@ bool Scheduler::try_rows(std::vector<PlanRow>& rows, std::vector<int32_t>& token
     tokens.insert(tokens.end(), r.tokens.begin() + cached, r.tokens.begin() + cached + n);
     used += n;
   }
-  return !rows.empty();
+  return rows.empty() ? 0 : 1;
 }
 
 PlanStatus Scheduler::plan(std::vector<PlanRow>& rows, std::vector<int32_t>& tokens) {
-  planned_.clear();
+  if (!planned_.empty()) {
+    rows.clear();
+    tokens.clear();
+    return PLAN_STEP_PENDING;
+  }
   if (live_.empty()) {
     rows.clear();
     tokens.clear();
     return PLAN_IDLE;
   }
   for (;;) {
-    if (try_rows(rows, tokens)) {
+    const int got = try_rows(rows, tokens);
+    if (got < 0) return PLAN_INTERNAL;
+    if (got > 0) {
       planned_ = rows;
       return PLAN_OK;
     }
@@ -117,14 +131,28 @@ PlanStatus Scheduler::plan(std::vector<PlanRow>& rows, std::vector<int32_t>& tok
   }
 }
 
-void Scheduler::commit(const int32_t* sampled, int n_sampled, std::vector<Emitted>& out) {
+int Scheduler::num_planned_samples() const {
+  int n = 0;
+  for (const PlanRow& row : planned_)
+    if (row.sample && live_.count(row.id)) n += 1;
+  return n;
+}
+
+void Scheduler::abort_step() {
+  for (const PlanRow& row : planned_)
+    if (live_.count(row.id)) cache_->abort_step(row.id);
+  planned_.clear();
+}
+
+bool Scheduler::commit(const int32_t* sampled, int n_sampled, std::vector<Emitted>& out) {
   out.clear();
+  if (n_sampled != num_planned_samples() || (n_sampled > 0 && sampled == nullptr)) return false;
   int k = 0;
   for (const PlanRow& row : planned_) {
     auto it = live_.find(row.id);
     if (it == live_.end()) continue;
     cache_->commit(row.id);
-    if (!row.sample || k >= n_sampled) continue;
+    if (!row.sample) continue;
     Request& r = it->second;
     const int32_t tok = sampled[k++];
     r.tokens.push_back(tok);
@@ -139,6 +167,7 @@ void Scheduler::commit(const int32_t* sampled, int n_sampled, std::vector<Emitte
     }
   }
   planned_.clear();
+  return true;
 }
 
 bool Scheduler::abort(RequestId id) {

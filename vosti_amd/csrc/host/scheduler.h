@@ -49,12 +49,15 @@ enum AdmissionStatus : int {
   TOO_MANY_EOS_TOKEN_IDS = 3,
   ZERO_MAX_TOKENS = 4,
   HISTORY_CAPACITY_OVERFLOW = 5,
+  EMPTY_EOS_TOKEN_IDS = 6,   // no end token although end tokens are not ignored (request_state.rs:207, engine.rs:2718-2720)
 };
 
 enum PlanStatus : int {
   PLAN_OK = 0,
   PLAN_IDLE = 1,          // nothing live
   PLAN_OUT_OF_PAGES = 2,  // a request cannot fit even the empty pool
+  PLAN_STEP_PENDING = 3,  // the step planned before was neither committed nor given up
+  PLAN_INTERNAL = 4,      // the cache manager refused a row for a reason other than pages: a fault of the engine
 };
 
 struct SchedulerConfig {
@@ -88,8 +91,13 @@ class Scheduler {
   // Decides the next step and takes its pages.  rows/tokens describe it:
   // tokens holds the rows' tokens back to back.
   PlanStatus plan(std::vector<PlanRow>& rows, std::vector<int32_t>& tokens);
-  // The planned step ran; `sampled` has one token per sampled row, in row order.
-  void commit(const int32_t* sampled, int n_sampled, std::vector<Emitted>& out);
+  // The planned step ran; `sampled` has one token per sampled row, in row order.  False, and nothing
+  // committed, if their number is not the number of sampled rows of the plan.
+  bool commit(const int32_t* sampled, int n_sampled, std::vector<Emitted>& out);
+  // The planned step did not run (a launch failed): the rows' tokens stay uncomputed, their pages stay
+  // with their requests, and the next plan() decides again.
+  void abort_step();
+  int num_planned_samples() const;
   // Gives up a live request (waiting or running).
   bool abort(RequestId id);
 
@@ -107,7 +115,7 @@ class Scheduler {
     std::vector<int32_t> eos;
     bool ignore_eos = false;
   };
-  bool try_rows(std::vector<PlanRow>& rows, std::vector<int32_t>& tokens);
+  int try_rows(std::vector<PlanRow>& rows, std::vector<int32_t>& tokens);   // 1: rows, 0: none fit, -1: fault
   int chunk_for(int remaining, int available, bool first) const;
   int page_debt() const;
 

@@ -45,6 +45,7 @@ class Engine:
         n = max_num_seqs + 1
         self.slot_temperature = np.zeros(n, dtype=np.float32)
         self.slot_seed = np.zeros(n, dtype=np.uint64)
+        self.slot_owner = np.full(n, -1, dtype=np.int64)      # the request whose state the slot holds
         self._params: dict[int, SamplingParams] = {}
         self._next_id = 0
         self.steps = 0
@@ -63,8 +64,9 @@ class Engine:
         vocab = self.model.spec.vocab_size
         if any((not isinstance(t, int)) or t < 0 or t >= vocab for t in prompt_ids):
             raise ValueError(f"prompt token outside [0, {vocab})")
+        # A request without end tokens runs to max_tokens.
         status = self.scheduler.add_request(request_id, list(prompt_ids), params.max_tokens, params.eos_token_ids,
-                                            params.ignore_eos)
+                                            params.ignore_eos or not params.eos_token_ids)
         if status != "Accepted":
             raise ValueError(f"request {request_id} refused: {status}")
         self._params[request_id] = params
@@ -80,6 +82,24 @@ class Engine:
         self.last_scheduled = [r.request_id for r in rows]
         if not rows:
             return {}
+        try:
+            sampled = self._forward_and_sample(rows)
+        except BaseException:
+            # Nothing of the step counts: the rows' tokens stay uncomputed, their pages stay with their
+            # requests, and the next plan() decides again.
+            self.scheduler.abort_step()
+            raise
+        emitted = self.scheduler.commit(sampled)
+        self.steps += 1
+        out = {}
+        for e in emitted:
+            out[e.request_id] = e.token
+            if e.finished:
+                self._params.pop(e.request_id, None)
+        return out
+
+    def _forward_and_sample(self, rows) -> list[int]:
+        """Runs the planned rows and draws one token per sampled row (one readback)."""
         entries = [StepEntry(r.request_id, r.tokens, [len(r.tokens) - 1] if r.sample else []) for r in rows]
         sampling = [r for r in rows if r.sample]
         logits = self.runner.run(entries)
@@ -93,11 +113,13 @@ class Engine:
             temps = np.zeros(len(sampling), dtype=np.float32)
             unis = np.zeros(len(sampling), dtype=np.float32)
             for i, r in enumerate(sampling):
-                p = self._params[r.request_id]
-                # The slot holds the request's sampler state; it is (re)written when the row is planned,
-                # since a request gets its slot at admission, inside plan().
-                self.slot_temperature[r.state_slot] = p.temperature
-                self.slot_seed[r.state_slot] = p.seed & ((1 << 64) - 1)
+                # The slot holds the request's sampler state.  A request gets its slot at admission, inside
+                # plan(), so the state is written when the request's first sampled row shows up in it.
+                if self.slot_owner[r.state_slot] != r.request_id:
+                    p = self._params[r.request_id]
+                    self.slot_owner[r.state_slot] = r.request_id
+                    self.slot_temperature[r.state_slot] = p.temperature
+                    self.slot_seed[r.state_slot] = p.seed & ((1 << 64) - 1)
                 temps[i] = self.slot_temperature[r.state_slot]
                 unis[i] = uniform_for(int(self.slot_seed[r.state_slot]), r.output_index)
             if (temps > 0).any():
@@ -106,14 +128,7 @@ class Engine:
             else:
                 ids = self.kernels.sample(logits)
             sampled = ids.cpu().tolist()     # the step's one synchronisation
-        emitted = self.scheduler.commit(sampled)
-        self.steps += 1
-        out = {}
-        for e in emitted:
-            out[e.request_id] = e.token
-            if e.finished:
-                self._params.pop(e.request_id, None)
-        return out
+        return sampled
 
     # ------------------------------------------------------------- generate
     def generate(self, prompts: list[list[int]], params: SamplingParams | list[SamplingParams] | None = None,

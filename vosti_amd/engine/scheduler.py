@@ -11,8 +11,12 @@ from ..cache.host import host_lib, i32_array
 from ..cache.manager import CacheManager, OutOfPages
 
 ADMISSION = ["Accepted", "DuplicateRequestId", "EmptyPrompt", "TooManyEosTokenIds", "ZeroMaxTokens",
-             "HistoryCapacityOverflow"]
-PLAN_OK, PLAN_IDLE, PLAN_OUT_OF_PAGES = 0, 1, 2
+             "HistoryCapacityOverflow", "EmptyEosTokenIds"]
+PLAN_OK, PLAN_IDLE, PLAN_OUT_OF_PAGES, PLAN_STEP_PENDING, PLAN_INTERNAL = 0, 1, 2, 3, 4
+
+
+class SchedulerError(RuntimeError):
+    """The scheduler was driven out of order, or found the cache manager in a state it cannot plan from."""
 
 
 @dataclass
@@ -46,8 +50,14 @@ class Scheduler:
         if h:
             self._lib.vh_sched_destroy(h)
 
-    def add_request(self, request_id: int, prompt: list[int], max_tokens: int, eos_token_ids=(), ignore_eos=False) -> str:
-        """Returns the admission status by name ('Accepted', 'EmptyPrompt', ...); only appends to the waiting queue."""
+    def add_request(self, request_id: int, prompt: list[int], max_tokens: int, eos_token_ids=(),
+                    ignore_eos: bool | None = None) -> str:
+        """Returns the admission status by name ('Accepted', 'EmptyPrompt', ...); only appends to the waiting queue.
+
+        ``ignore_eos`` None: end tokens count if there are any.  False with no end token is refused as
+        'EmptyEosTokenIds', as the reference refuses it (src/exec/engine.rs:2718-2720)."""
+        if ignore_eos is None:
+            ignore_eos = not eos_token_ids
         if len(eos_token_ids) > 3:
             return "TooManyEosTokenIds"
         st = self._lib.vh_sched_add_request(self._h, request_id, i32_array(prompt) if prompt else None, len(prompt),
@@ -61,6 +71,10 @@ class Scheduler:
         st = self._lib.vh_sched_plan(self._h, ctypes.byref(n_rows), ctypes.byref(n_tokens))
         if st == PLAN_OUT_OF_PAGES:
             raise OutOfPages("a request needs more cache pages than the pool has, even alone")
+        if st == PLAN_STEP_PENDING:
+            raise SchedulerError("plan() before the step planned last was committed or given up (abort_step)")
+        if st == PLAN_INTERNAL:
+            raise SchedulerError("the cache manager refused a planned row for a reason other than pages")
         if st == PLAN_IDLE or n_rows.value == 0:
             return []
         rows = np.empty((n_rows.value, 6), dtype=np.int64)
@@ -73,11 +87,19 @@ class Scheduler:
         return out
 
     def commit(self, sampled: list[int]) -> list[Emitted]:
+        """The planned step ran: one sampled token per sampled row, in row order."""
         n = self._lib.vh_sched_commit(self._h, i32_array(sampled) if sampled else None, len(sampled))
+        if n < 0:
+            raise SchedulerError(f"commit() got {len(sampled)} sampled tokens for a plan with "
+                                 f"{self._lib.vh_sched_num_planned_samples(self._h)} sampled rows; nothing was committed")
         out = np.empty((n, 3), dtype=np.int64)
         if n:
             self._lib.vh_sched_get_emitted(self._h, out.ctypes.data)
         return [Emitted(r, t, bool(f)) for r, t, f in out.tolist()]
+
+    def abort_step(self) -> None:
+        """The planned step did not run: its rows' tokens stay uncomputed and the next plan() decides again."""
+        self._lib.vh_sched_abort_step(self._h)
 
     def abort(self, request_id: int) -> bool:
         return bool(self._lib.vh_sched_abort(self._h, request_id))

@@ -16,20 +16,41 @@ replayed from then on.
 """
 from __future__ import annotations
 
+from collections import OrderedDict
 from dataclasses import dataclass, field
 
 import numpy as np
 import torch
 
 from ..cache import CachePool
-from ..kernels.ops import ATTN_ITEM_ROWS, SEGMENT_KEYS
-from ..parts.base import GroupTables, StepContext
+from ..parts.base import GroupTables, HostStep, StepContext
 
-WIDTH_BUCKET = 8       # captured block tables grow in steps of this many pages
 # Captured decode steps have one of these numbers of rows; a step with fewer is filled up with rows that
 # read one key of page 0 and write nothing (the reference pads its graphs likewise,
-# python/vosti_kernels/graph_overlay.py:177-389).
+# python/vosti_kernels/graph_overlay.py:177-389).  Block tables are captured with one of these widths
+# times eight pages, so that a long generation walks through few captures.
 ROW_BUCKETS = (1, 2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64, 96, 128, 192, 256, 384, 512)
+WIDTH_STEP = 8
+MAX_GRAPHS = 24        # captured graphs kept; the least recently replayed one goes first
+
+
+def _bucket(n: int) -> int:
+    """The smallest of 1, 2, 3, 4, 6, 8, 12, 16, ... that is at least n."""
+    b = 1
+    while True:
+        for m in (b, b + b // 2):
+            if m >= n and (m == b or b >= 2):
+                return m
+        b *= 2
+
+
+def width_bucket(pages: int) -> int:
+    return WIDTH_STEP * _bucket(-(-max(pages, 1) // WIDTH_STEP))
+
+
+class GraphError(RuntimeError):
+    """A capture or a replay failed: the runner replays nothing any more
+    (python/vosti_kernels/graph_overlay.py:120-124, 173-175: no eager fallback after a failed replay)."""
 
 
 @dataclass
@@ -43,16 +64,17 @@ class StepEntry:
 class _Layout:
     """Host arrays of one step and where each lies in the one buffer that is uploaded."""
     parts: list[np.ndarray]
+    names: list[str]            # names of the arrays that parts asked for (after the fixed ones)
     offsets: list[int]
     total: int
-    q_lens: list[int]
-    starts: list[int]
-    max_k_len: int
-    max_decode_k_len: int
+    host: HostStep
 
     def pack(self, out: np.ndarray) -> None:
         for p, o in zip(self.parts, self.offsets):
             out[o:o + p.size] = p.reshape(-1)
+
+
+N_FIXED = 6      # ids, positions, cu_q, k_len, state slots, wanted rows
 
 
 @dataclass
@@ -62,30 +84,41 @@ class _Captured:
     staging: torch.Tensor     # pinned host twin
     logits: torch.Tensor      # the graph's output
     copied: torch.cuda.Event  # the last upload from ``staging``
+    workspace: torch.Tensor   # the buffer its launches point into
 
 
 class ModelRunner:
     """Binds a model to a cache pool and runs steps."""
 
-    def __init__(self, model, pool: CachePool, graphs: bool = False):
+    def __init__(self, model, pool: CachePool, graphs: bool = False, max_graphs: int = MAX_GRAPHS):
         self.model, self.pool, self.cache = model, pool, pool.manager
         self.kernels = model.kernels
         self.graphs = graphs
-        self._scratch: torch.Tensor | None = None
+        self.max_graphs = max(1, int(max_graphs))
+        self._workspace: torch.Tensor | None = None
         self._seen: set[tuple] = set()
-        self._captured: dict[tuple, _Captured] = {}
-        self._keepalive: list[torch.Tensor] = []
-        self.graph_stats = {"eager": 0, "captured": 0, "replayed": 0}
+        self._captured: "OrderedDict[tuple, _Captured]" = OrderedDict()
+        self._graph_pool = None
+        self._poisoned: str | None = None
+        self.graph_stats = {"eager": 0, "captured": 0, "replayed": 0, "evicted": 0}
+        # What the parts want of every step: one provider per distinct kind of per-step arrays.
+        self._parts = list(model.parts())
+        self._providers = {}
+        for part in self._parts:
+            if part.step_inputs_key is not None:
+                self._providers.setdefault(part.step_inputs_key, part)
 
     # ---------------------------------------------------------------- pieces
-    def _attn_scratch(self, n_floats: int) -> torch.Tensor:
-        if self._scratch is None or self._scratch.numel() < n_floats:
+    def _get_workspace(self, n_floats: int) -> torch.Tensor:
+        if self._workspace is None or self._workspace.numel() < n_floats:
             if torch.cuda.is_current_stream_capturing():
-                raise RuntimeError("the attention scratch buffer must be sized before a graph is captured")
-            if self._scratch is not None and self._captured:
-                self._keepalive.append(self._scratch)      # captured graphs still point at it
-            self._scratch = torch.empty(max(n_floats, 1 << 16), dtype=torch.float32, device="cuda")
-        return self._scratch
+                raise RuntimeError("a part asks for more workspace inside a capture than it announced before it")
+            # Captured graphs keep the buffer they were recorded with (``_Captured.workspace``).
+            self._workspace = torch.empty(max(n_floats, 1 << 16), dtype=torch.float32, device="cuda")
+        return self._workspace
+
+    def workspace_needed(self, host: HostStep) -> int:
+        return max((p.workspace_floats(host) for p in self._parts), default=0)
 
     def begin(self, entries: list[StepEntry]) -> None:
         """Takes the pages of the step's tokens (and a state slot for new requests)."""
@@ -107,10 +140,12 @@ class ModelRunner:
         for e in entries:
             self.cache.commit(e.request_id)
 
-    def _layout(self, entries: list[StepEntry], widths: list[int] | None = None, rows: int | None = None) -> _Layout:
+    def _layout(self, entries: list[StepEntry], widths: list[int] | None = None, rows: int | None = None,
+                bound: int | None = None) -> _Layout:
         """The step's host arrays.  ``widths``: block-table width per group (default: what the step needs).
         ``rows``: fill up to this many sequences with padding rows of one token: token 0 at position 0,
-        one key (whatever page 0 holds), slot -1 (nothing is stored), logits wanted like the others."""
+        one key (whatever page 0 holds), slot -1 (nothing is stored), logits wanted like the others.
+        ``bound``: the step is recorded for replay and its launches must cover this many keys."""
         cache, spec = self.cache, self.model.spec
         real = len(entries)
         S = max(real, rows or 0)
@@ -126,13 +161,13 @@ class ModelRunner:
         ids = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries] + [np.zeros(S - real, dtype=np.int64)])
         if ids.min() < 0 or ids.max() >= spec.vocab_size:
             raise ValueError(f"token id out of range [0, {spec.vocab_size})")
-        k_len = np.asarray([s + n for s, n in zip(starts, q_lens)], dtype=np.int32)
-        if int(k_len.max()) > spec.max_positions:
-            raise ValueError(f"a request would reach {int(k_len.max())} tokens; the model's positions end at {spec.max_positions}")
+        k_lens = [s + n for s, n in zip(starts, q_lens)]
+        if max(k_lens) > spec.max_positions:
+            raise ValueError(f"a request would reach {max(k_lens)} tokens; the model's positions end at {spec.max_positions}")
         positions = np.concatenate([np.arange(s, s + n, dtype=np.int32) for s, n in zip(starts, q_lens)])
         cu_q = np.zeros(S + 1, dtype=np.int32)
         np.cumsum(q_lens, out=cu_q[1:])
-        state_slots = np.asarray([cache.state_slot(e.request_id) for e in entries] + [0] * (S - real), dtype=np.int32)
+        state_slots = [cache.state_slot(e.request_id) for e in entries] + [0] * (S - real)
         want = []
         for e, base, n in zip(entries, cu_q[:-1], q_lens):
             for w in e.want:
@@ -140,16 +175,10 @@ class ModelRunner:
                     raise ValueError(f"request {e.request_id}: wanted place {w} is outside its {n} tokens")
                 want.append(int(base) + w)
         want += [int(cu_q[s]) for s in range(real, S)]
-        prefill_items, decode_items = [], []
-        for s, n in enumerate(q_lens):
-            if n == 1:
-                decode_items.append((s, 0))
-            else:
-                prefill_items.extend((s, off) for off in range(0, n, ATTN_ITEM_ROWS))
-        parts: list[np.ndarray] = [ids.astype(np.int32), positions, cu_q, k_len, state_slots,
-                                   np.asarray(want, dtype=np.int32),
-                                   np.asarray(prefill_items, dtype=np.int32).reshape(-1, 2),
-                                   np.asarray(decode_items, dtype=np.int32).reshape(-1, 2)]
+        host = HostStep(q_lens=q_lens, starts=starts, k_lens=k_lens, state_slots=state_slots,
+                        k_len_bound=bound if bound is not None else max(k_lens), frozen=bound is not None)
+        parts: list[np.ndarray] = [ids.astype(np.int32), positions, cu_q, np.asarray(k_lens, dtype=np.int32),
+                                   np.asarray(state_slots, dtype=np.int32), np.asarray(want, dtype=np.int32)]
         for g in range(len(self.pool.group_windows)):
             width = widths[g] if widths else self.needed_width(entries, g)
             table = np.zeros((S, width), dtype=np.int32)
@@ -158,27 +187,33 @@ class ModelRunner:
                 cache.block_table_row(e.request_id, g, width, table[s])
                 cache.slots(e.request_id, g, starts[s], q_lens[s], slots[cu_q[s]:cu_q[s + 1]])
             parts += [slots, table]
+        names: list[str] = []
+        for provider in self._providers.values():
+            for name, arr in provider.step_inputs(host).items():
+                if name in names:
+                    raise ValueError(f"two parts ask for a per-step array named {name!r}")
+                names.append(name)
+                parts.append(np.ascontiguousarray(arr, dtype=np.int32))
         # One buffer, one copy; every piece starts on a 16-byte boundary.
         offsets, total = [], 0
         for p in parts:
             offsets.append(total)
             total += (p.size + 3) & ~3
-        dec_k = [int(k_len[s]) for s, n in enumerate(q_lens) if n == 1]
-        return _Layout(parts, offsets, max(total, 4), q_lens, starts, int(k_len.max()), max(dec_k) if dec_k else 0)
+        return _Layout(parts, names, offsets, max(total, 4), host)
 
     def needed_width(self, entries: list[StepEntry], group: int) -> int:
         return max(1, max(self.cache.num_logical_pages(e.request_id, group) for e in entries))
 
-    def _context(self, lay: _Layout, dev: torch.Tensor, max_k_len: int, max_decode_k_len: int):
+    def _context(self, lay: _Layout, dev: torch.Tensor):
         views = [dev[o:o + p.size].view(p.shape) for p, o in zip(lay.parts, lay.offsets)]
-        ids_d, pos_d, cu_d, klen_d, slots_d, want_d, pre_d, dec_d = views[:8]
-        groups = [GroupTables(slots=views[8 + 2 * g], block_table=views[9 + 2 * g], window=w)
+        ids_d, pos_d, cu_d, klen_d, slots_d, want_d = views[:N_FIXED]
+        n_groups = len(self.pool.group_windows)
+        groups = [GroupTables(slots=views[N_FIXED + 2 * g], block_table=views[N_FIXED + 1 + 2 * g], window=w)
                   for g, w in enumerate(self.pool.group_windows)]
-        ctx = StepContext(kernels=self.kernels, num_tokens=sum(lay.q_lens), num_seqs=len(lay.q_lens), positions=pos_d,
-                          cu_q=cu_d, k_len=klen_d, state_slots=slots_d, groups=groups, prefill_items=pre_d,
-                          decode_items=dec_d, max_k_len=max_k_len, max_decode_k_len=max_decode_k_len,
-                          host_q_lens=lay.q_lens, host_starts=lay.starts, host_state_slots=lay.parts[4].tolist(),
-                          attn_scratch=self._attn_scratch)
+        inputs = dict(zip(lay.names, views[N_FIXED + 2 * n_groups:]))
+        ctx = StepContext(kernels=self.kernels, num_tokens=sum(lay.host.q_lens), num_seqs=len(lay.host.q_lens),
+                          positions=pos_d, cu_q=cu_d, k_len=klen_d, state_slots=slots_d, groups=groups, host=lay.host,
+                          inputs=inputs, workspace=self._get_workspace)
         return ids_d, ctx, want_d
 
     def build_context(self, entries: list[StepEntry]):
@@ -186,21 +221,25 @@ class ModelRunner:
         lay = self._layout(entries)
         host = np.zeros(lay.total, dtype=np.int32)
         lay.pack(host)
-        return self._context(lay, torch.from_numpy(host).to("cuda"), lay.max_k_len, lay.max_decode_k_len)
+        return self._context(lay, torch.from_numpy(host).to("cuda"))
 
     # ---------------------------------------------------------------- running
     def run(self, entries: list[StepEntry]) -> torch.Tensor:
         """The forward pass of a step whose pages are taken; logits [wanted, vocab] in the element type."""
         if self.graphs and all(len(e.tokens) == 1 and e.want == [0] for e in entries):
             return self._run_decode_graph(entries)
+        return self._run_eager(entries)
+
+    def _run_eager(self, entries: list[StepEntry]) -> torch.Tensor:
         self.graph_stats["eager"] += 1
         ids, ctx, want = self.build_context(entries)
         return self.model.forward(ids, ctx, self.pool.entries, want)
 
     def _run_decode_graph(self, entries: list[StepEntry]) -> torch.Tensor:
+        if self._poisoned is not None:
+            raise GraphError(f"graph replay is switched off after a failure: {self._poisoned}")
         P = self.pool.page_size
-        widths = [-(-self.needed_width(entries, g) // WIDTH_BUCKET) * WIDTH_BUCKET
-                  for g in range(len(self.pool.group_windows))]
+        widths = [width_bucket(self.needed_width(entries, g)) for g in range(len(self.pool.group_windows))]
         # A mixer with state of its own would have to be told which rows are padding: no padding then.
         rows = len(entries) if self.pool.has_state else next((b for b in ROW_BUCKETS if b >= len(entries)), len(entries))
         key = (rows, tuple(widths))
@@ -208,44 +247,49 @@ class ModelRunner:
         if cap is None and key not in self._seen:
             # First sight of a signature: eagerly, which also warms up every kernel it uses.
             self._seen.add(key)
-            self.graph_stats["eager"] += 1
-            ids, ctx, want = self.build_context(entries)
-            return self.model.forward(ids, ctx, self.pool.entries, want)
-        lay = self._layout(entries, widths, rows)
+            return self._run_eager(entries)
         # Launch geometry is frozen in the graph: it must cover every length the tables can hold.
         cover = min(max(widths) * P, self.model.spec.max_positions)
-        if cap is None:
-            self._attn_scratch(self._max_scratch(rows, cover))
-            staging = torch.empty(lay.total, dtype=torch.int32, pin_memory=True)
-            meta = torch.zeros(lay.total, dtype=torch.int32, device="cuda")
-            lay.pack(staging.numpy())
-            meta.copy_(staging, non_blocking=True)
-            ids, ctx, want = self._context(lay, meta, cover, cover)
-            torch.cuda.synchronize()
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                logits = self.model.forward(ids, ctx, self.pool.entries, want)
-            cap = _Captured(graph, meta, staging, logits, torch.cuda.Event())
-            self._captured[key] = cap
-            self.graph_stats["captured"] += 1
-        else:
-            cap.copied.synchronize()                       # the staging buffer is free again
-            lay.pack(cap.staging.numpy())
-            cap.meta.copy_(cap.staging, non_blocking=True)
-        cap.copied.record()
-        cap.graph.replay()
+        lay = self._layout(entries, widths, rows, bound=cover)
+        try:
+            if cap is None:
+                cap = self._capture(key, lay)
+            else:
+                self._captured.move_to_end(key)
+                cap.copied.synchronize()                       # the staging buffer is free again
+                lay.pack(cap.staging.numpy())
+                cap.meta.copy_(cap.staging, non_blocking=True)
+            cap.copied.record()
+            cap.graph.replay()
+        except Exception as e:
+            self._poisoned = f"{type(e).__name__}: {e}"
+            self._captured.clear()
+            raise GraphError(f"graph capture or replay failed ({self._poisoned}); no further step is replayed") from e
         self.graph_stats["replayed"] += 1
         return cap.logits[:len(entries)]
 
-    def _max_scratch(self, tokens: int, cover: int) -> int:
-        """Floats of attention scratch that any mixer of the model needs for ``tokens`` decode rows over ``cover`` keys."""
-        nseg = -(-cover // SEGMENT_KEYS)
-        need = 1
-        for block in self.model.layers:
-            m = block.mixer
-            if hasattr(m, "nq") and hasattr(m, "d"):
-                need = max(need, self.kernels.attn_scratch_floats(tokens, m.nq, m.d, nseg))
-        return need
+    def _capture(self, key: tuple, lay: _Layout) -> _Captured:
+        while len(self._captured) >= self.max_graphs:
+            self._captured.popitem(last=False)                 # the least recently replayed
+            self.graph_stats["evicted"] += 1
+        workspace = self._get_workspace(self.workspace_needed(lay.host))
+        staging = torch.empty(lay.total, dtype=torch.int32, pin_memory=True)
+        meta = torch.zeros(lay.total, dtype=torch.int32, device="cuda")
+        lay.pack(staging.numpy())
+        meta.copy_(staging, non_blocking=True)
+        ids, ctx, want = self._context(lay, meta)
+        torch.cuda.synchronize()
+        if self._graph_pool is None:
+            # One memory pool for all captures: they never replay at the same time, so the
+            # intermediates of one may lie where another's lay; each keeps its own logits.
+            self._graph_pool = torch.cuda.graph_pool_handle()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, pool=self._graph_pool):
+            logits = self.model.forward(ids, ctx, self.pool.entries, want)
+        cap = _Captured(graph, meta, staging, logits, torch.cuda.Event(), workspace)
+        self._captured[key] = cap
+        self.graph_stats["captured"] += 1
+        return cap
 
     # ------------------------------------------------------------------ whole
     def step(self, entries: list[StepEntry]) -> torch.Tensor:

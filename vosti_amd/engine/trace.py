@@ -17,6 +17,11 @@ def build_parser() -> argparse.ArgumentParser:
                    help="most tokens live requests hold at any time, each request rounded up to a page")
     p.add_argument("--page-size", type=int, default=64, help="tokens per cache page (a power of two, default 64)")
     p.add_argument("--max-requests", type=int, default=8, help="most requests alive at a time (state slots)")
+    p.add_argument("--prefix-cache", action="store_true",
+                   help="a request whose first tokens equal full pages that an earlier request left reuses those pages: "
+                        "feed such a request its tokens from the first uncached one on (--prefix-report tells which)")
+    p.add_argument("--prefix-report", default=None,
+                   help="a file that gets one line '<id> <cached tokens>' when a request with a 'prompt' field is first seen")
     return p
 
 
@@ -36,8 +41,10 @@ def main(argv: list[str] | None = None) -> int:
     model = load_model(args.model, args.dtype)
     page = args.page_size
     num_pages = max(1, -(-args.max_tokens // page))
-    pool = CachePool(model, page_size=page, num_pages=num_pages, num_slots=args.max_requests)
+    pool = CachePool(model, page_size=page, num_pages=num_pages, num_slots=args.max_requests,
+                     prefix_cache=args.prefix_cache)
     runner = ModelRunner(model, pool)
+    report = open(args.prefix_report, "a") if args.prefix_report else None
     out_dir = Path(args.out)
     out_dir.mkdir(parents=True, exist_ok=True)
     ids: dict[str, int] = {}     # request names -> numbers; a name may come back after it ended
@@ -55,6 +62,17 @@ def main(argv: list[str] | None = None) -> int:
             if name not in ids:
                 ids[name] = next_id
                 next_id += 1
+                if args.prefix_cache and "prompt" in e:
+                    # The whole prompt is announced so that cached pages can be matched; the entry's tokens
+                    # must then start right after the cached ones, which are not computed again.
+                    cached = runner.cache.add_request(ids[name], [int(t) for t in e["prompt"]])
+                    if report:
+                        report.write(f"{name} {cached}\n")
+                        report.flush()
+                    skip = cached - int(e.get("start", 0))
+                    if skip < 0:
+                        raise SystemExit(f"trace_run: request {name} starts at {e.get('start', 0)} but {cached} tokens are cached")
+                    e = dict(e, tokens=e["tokens"][skip:], want=[w - skip for w in e.get("want", []) if w >= skip])
             entries.append(StepEntry(ids[name], [int(t) for t in e["tokens"]], [int(w) for w in e.get("want", [])]))
         logits = runner.step(entries)
         if logits.shape[0] > 0:

@@ -15,7 +15,7 @@ import torch
 
 from . import build
 
-ABI_VERSION = 10
+ABI_VERSION = 11
 SEGMENT_KEYS = 256
 ATTN_ITEM_ROWS = 128      # rows of one prompt item of paged_attention
 
@@ -276,8 +276,9 @@ class Kernels:
                    self._stream())
         return q_out
 
-    def attn_scratch_floats(self, tokens: int, nq: int, d: int, nseg: int) -> int:
-        return int(self.lib.vk_attn_scratch_floats(tokens, nq, d, nseg))
+    def attn_scratch_floats(self, items: int, nq: int, d: int, nseg: int) -> int:
+        """float32 elements of scratch that decode attention (mode 1) needs for ``items`` decoded tokens."""
+        return int(self.lib.vk_attn_scratch_floats(items, nq, d, nseg))
 
     def paged_attention(self, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                         block_table: torch.Tensor, cu_q: torch.Tensor, k_len: torch.Tensor, items: torch.Tensor,
@@ -287,9 +288,9 @@ class Kernels:
         """Attention of the rows named by ``items`` over the paged cache (see attention.hip).
 
         items [n, 2] = (sequence, first row).  mode 0: an item is up to ATTN_ITEM_ROWS consecutive new
-        rows of its sequence; mode 2: the same through the kernel that takes every shape (same bits);
-        mode 1: an item is a single decoded token.  ``max_k_len`` is the host's bound on k_len; the
-        block table must cover it."""
+        rows of its sequence; modes 2 and 6: the same through a named kernel (same bits); mode 1: an item
+        is a single decoded token; modes 3, 4, 5: the same through a named kernel (same bits; see
+        attention.hip).  ``max_k_len`` is the host's bound on k_len; the block table must cover it."""
         T, nq, d = q.shape
         pages, nkv, P, d2 = k_cache.shape
         S, W = block_table.shape
@@ -306,11 +307,11 @@ class Kernels:
         out = torch.empty_like(q) if out is None else out
         self._elem(out, "out", T, nq, d)
         sp = None
-        if mode == 1:
+        if mode in (1, 3, 4, 5):
             need_seg = -(-max_k_len // SEGMENT_KEYS)
             if nseg < need_seg:
                 raise KernelError(f"attention: {nseg} segments do not cover {max_k_len} keys")
-            need = self.attn_scratch_floats(T, nq, d, nseg)
+            need = self.attn_scratch_floats(n_items, nq, d, nseg)
             if scratch is None or scratch.numel() < need:
                 raise KernelError(f"attention: scratch of {need} floats needed")
             sp = self._f32(scratch, "scratch")

@@ -42,7 +42,12 @@ import sys
 import time
 from pathlib import Path
 
-FAMILIES = {"qwen3": "Qwen3ForCausalLM"}
+
+
+def families() -> dict[str, str]:
+    """--family names: the ``model_type`` of every registered architecture -> its name."""
+    from .config.registry import model_types
+    return model_types()
 
 
 def _env(name: str, default=None):
@@ -121,7 +126,7 @@ def run_engine(argv: list[str], family: str) -> int:
         raise SystemExit(f"device {args.device!r}: this engine runs on cuda:0 only")
     from .config import load_config
     cfg = load_config(args.model_path)
-    if cfg.architecture != FAMILIES[family]:
+    if cfg.architecture != families()[family]:
         raise SystemExit(f"{args.model_path} holds a {cfg.architecture}, not a {family} model")
     from .engine import Engine
     from .sampling import SamplingParams
@@ -190,7 +195,7 @@ def run_random_model(argv: list[str], family: str) -> int:
     from .config import config_from_dict
     from .weights import write_random_model
     raw = json.loads(Path(args.config).read_text())
-    raw.setdefault("architectures", [FAMILIES[family]])
+    raw.setdefault("architectures", [families()[family]])
     out = write_random_model(config_from_dict(raw), args.seed, args.out, getattr(torch, args.dtype))
     print(f"wrote {out}")
     return 0
@@ -199,7 +204,7 @@ def run_random_model(argv: list[str], family: str) -> int:
 def main(argv: list[str] | None = None) -> int:
     p = argparse.ArgumentParser(description="Launch the engine or write a random-weights model folder.")
     p.add_argument("--kind", required=True, choices=("engine", "random-model"))
-    p.add_argument("--family", required=True, choices=sorted(FAMILIES))
+    p.add_argument("--family", required=True, choices=sorted(families()))
     p.add_argument("args", nargs=argparse.REMAINDER, help="options of the chosen kind, after --")
     ns = p.parse_args(argv)
     rest = ns.args[1:] if ns.args[:1] == ["--"] else ns.args

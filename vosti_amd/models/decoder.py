@@ -7,6 +7,7 @@ layers, final norm, row selection before the vocabulary projection).
 """
 from __future__ import annotations
 
+from dataclasses import dataclass, field
 from typing import Iterator, Mapping
 
 import torch
@@ -36,6 +37,19 @@ def walk_params(part: Part, prefix: str = "") -> Iterator[tuple[str, Part, str, 
         yield from walk_params(child, f"{prefix}{name}.")
 
 
+@dataclass
+class ExpectedTensor:
+    """A tensor of the weight files: its shape and type rules, and every (part, local name) that gets it."""
+    spec: ParamSpec
+    owners: list[tuple[Part, str]] = field(default_factory=list)
+
+
+def walk_parts(part: Part) -> Iterator[Part]:
+    yield part
+    for child in part.children().values():
+        yield from walk_parts(child)
+
+
 class DecoderModel:
     def __init__(self, spec: ModelSpec, kernels: Kernels):
         spec.validate()
@@ -48,15 +62,25 @@ class DecoderModel:
         self.loaded = False
 
     # ------------------------------------------------------------ weights
-    def expected_tensors(self) -> dict[str, tuple[Part, str, ParamSpec]]:
-        """Tensor name in the weight files -> (owning part, its local name, spec)."""
-        out: dict[str, tuple[Part, str, ParamSpec]] = {}
+    def parts(self) -> Iterator[Part]:
+        """Every part of the model, sub-parts included."""
+        for root in (self.embedding, *self.layers, self.final_norm, self.head):
+            yield from walk_parts(root)
+
+    def expected_tensors(self) -> dict[str, ExpectedTensor]:
+        """Tensor name in the weight files -> what it must look like and which parts get it.  Parameters
+        that the specification gives the same tensor name share one tensor."""
+        out: dict[str, ExpectedTensor] = {}
 
         def add(names: Mapping[str, str], root: Part, prefix: str):
             for path, owner, local, ps in walk_params(root, prefix):
                 if path not in names:
                     raise ValueError(f"the configuration gives no tensor name for parameter {path!r}")
-                out[names[path]] = (owner, local, ps)
+                e = out.setdefault(names[path], ExpectedTensor(ps))
+                if tuple(e.spec.shape) != tuple(ps.shape):
+                    raise ValueError(f"tensor {names[path]!r} is shared by parameters of different shapes: "
+                                     f"{list(e.spec.shape)} and {list(ps.shape)} ({path!r})")
+                e.owners.append((owner, local))
 
         add(self.spec.names, self.embedding, "embedding.")
         add(self.spec.names, self.final_norm, "final_norm.")
@@ -68,12 +92,11 @@ class DecoderModel:
     def load_tensors(self, tensors: Mapping[str, torch.Tensor]) -> None:
         """``tensors``: file name -> GPU tensor, already checked against ``expected_tensors``."""
         per_part: dict[int, tuple[Part, dict[str, torch.Tensor]]] = {}
-        for name, (owner, local, _) in self.expected_tensors().items():
-            per_part.setdefault(id(owner), (owner, {}))[1][local] = tensors[name]
+        for name, e in self.expected_tensors().items():
+            for owner, local in e.owners:
+                per_part.setdefault(id(owner), (owner, {}))[1][local] = tensors[name]
         for owner, group in per_part.values():
             owner.load(group)
-        if getattr(self.head, "tied", False):
-            self.head.weight = self.embedding.weight
         self.loaded = True
 
     # ------------------------------------------------------------- caches

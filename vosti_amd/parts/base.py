@@ -13,8 +13,9 @@ To add a part, subclass the category's base class, decorate it with
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Any, Mapping
+from typing import Any, Callable, Mapping
 
+import numpy as np
 import torch
 
 from ..config.spec import PartSpec
@@ -98,8 +99,31 @@ class GroupTables:
 
 
 @dataclass
+class HostStep:
+    """One step as the host knows it: what parts may size launches and buffers by.
+
+    ``frozen``: the step's launches are recorded for replay with other lengths, so
+    their geometry must cover every key count up to ``k_len_bound`` (what the block
+    tables can hold); otherwise ``k_len_bound`` is the largest of ``k_lens``.
+    ``memo`` is a scratch pad for what a part derives from these lists, so that the
+    layers of a model that share a part kind derive it once per step."""
+    q_lens: list[int]           # tokens of each sequence in this step
+    starts: list[int]           # position of each sequence's first token in this step
+    k_lens: list[int]           # keys of each sequence once this step's tokens are stored
+    state_slots: list[int]      # the state slot of each sequence
+    k_len_bound: int
+    frozen: bool = False
+    memo: dict = field(default_factory=dict)
+
+
+@dataclass
 class StepContext:
-    """Everything about one step that parts may need.  Device tensors are int32."""
+    """Everything about one step that parts may need.  Device tensors are int32.
+
+    ``inputs`` holds the per-step device arrays that parts asked for through
+    ``Part.step_inputs`` (they travel in the step's one upload); ``workspace(n)``
+    gives a float32 buffer of at least n elements whose contents do not outlive a
+    part's forward (its size was announced through ``Part.workspace_floats``)."""
     kernels: Kernels
     num_tokens: int
     num_seqs: int
@@ -108,14 +132,22 @@ class StepContext:
     k_len: torch.Tensor          # [S]: keys of each sequence once this step's tokens are stored
     state_slots: torch.Tensor    # [S]: the state slot of each sequence
     groups: list[GroupTables]
-    prefill_items: torch.Tensor  # [n, 2]: (sequence, first row) of blocks of ATTN_ITEM_ROWS rows of multi-token sequences
-    decode_items: torch.Tensor   # [n, 2]: single-token sequences
-    max_k_len: int               # host copies, for launch geometry
-    max_decode_k_len: int
-    host_q_lens: list[int] = field(default_factory=list)
-    host_starts: list[int] = field(default_factory=list)   # position of each sequence's first token in this step
-    host_state_slots: list[int] = field(default_factory=list)   # host copy of ``state_slots``
-    attn_scratch: Any = None     # callable(n_floats) -> float32 tensor
+    host: HostStep
+    inputs: Mapping[str, torch.Tensor] = field(default_factory=dict)
+    workspace: Callable[[int], torch.Tensor] | None = None
+
+    # Host copies, for parts that loop over sequences on the host.
+    @property
+    def host_q_lens(self) -> list[int]:
+        return self.host.q_lens
+
+    @property
+    def host_starts(self) -> list[int]:
+        return self.host.starts
+
+    @property
+    def host_state_slots(self) -> list[int]:
+        return self.host.state_slots
 
 
 # ----------------------------------------------------------------- interfaces
@@ -135,6 +167,19 @@ class Part:
     def children(self) -> Mapping[str, "Part"]:
         """Sub-parts whose parameters live under ``<name>.`` of this part's names."""
         return {}
+
+    # Per-step needs beyond the context's own fields.  Parts with the same ``step_inputs_key`` get one
+    # shared set of arrays: the step function asks one of them and uploads the answer with the step.
+    step_inputs_key: str | None = None
+
+    def step_inputs(self, step: HostStep) -> Mapping[str, np.ndarray]:
+        """int32 host arrays this part wants on the GPU for the step, by name (``ctx.inputs[name]``).
+        Their shapes may depend on the number of sequences and tokens only when ``step.frozen``."""
+        return {}
+
+    def workspace_floats(self, step: HostStep) -> int:
+        """float32 elements of ``ctx.workspace`` that this part's forward will ask for in this step."""
+        return 0
 
 
 class Norm(Part):

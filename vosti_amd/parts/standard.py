@@ -7,11 +7,12 @@ from __future__ import annotations
 
 from typing import Mapping
 
+import numpy as np
 import torch
 
 from ..config.spec import PartSpec
-from ..kernels.ops import Kernels, SEGMENT_KEYS
-from .base import (Block, Embedding, FeedForward, Head, KVPagesSpec, Mixer, Norm, PagedKV, ParamSpec, Part,
+from ..kernels.ops import ATTN_ITEM_ROWS, Kernels, SEGMENT_KEYS
+from .base import (Block, Embedding, FeedForward, Head, HostStep, KVPagesSpec, Mixer, Norm, PagedKV, ParamSpec, Part,
                    PositionEncoding, StepContext, build_part, register_part)
 
 
@@ -160,6 +161,42 @@ class Attention(Mixer):
     def cache_spec(self):
         return KVPagesSpec(self.nkv, self.d, self.window)
 
+    # The attention kernels work on items: a single decoded token, or up to ATTN_ITEM_ROWS consecutive rows
+    # of a sequence that brings several tokens.  The item lists are the same for every attention layer.
+    step_inputs_key = "attention.items"
+
+    @staticmethod
+    def _items(step: HostStep) -> dict:
+        m = step.memo.get("attention.items")
+        if m is None:
+            prefill, decode, decode_keys = [], [], 0
+            for s, n in enumerate(step.q_lens):
+                if n == 1:
+                    decode.append((s, 0))
+                    decode_keys = max(decode_keys, step.k_lens[s])
+                else:
+                    prefill.extend((s, off) for off in range(0, n, ATTN_ITEM_ROWS))
+            # Recorded launches must cover every length that the tables can hold.
+            bound = step.k_len_bound if step.frozen else decode_keys
+            m = {"prefill": prefill, "decode": decode, "decode_bound": bound, "nseg": -(-bound // SEGMENT_KEYS)}
+            step.memo["attention.items"] = m
+        return m
+
+    @classmethod
+    def _items_arrays(cls, step: HostStep) -> dict:
+        m = cls._items(step)
+        return {"attention.prefill_items": np.asarray(m["prefill"], dtype=np.int32).reshape(-1, 2),
+                "attention.decode_items": np.asarray(m["decode"], dtype=np.int32).reshape(-1, 2)}
+
+    def step_inputs(self, step: HostStep):
+        return self._items_arrays(step)
+
+    def workspace_floats(self, step: HostStep) -> int:
+        m = self._items(step)
+        if not m["decode"]:
+            return 0
+        return self.kernels.attn_scratch_floats(len(m["decode"]), self.nq, self.d, m["nseg"])
+
     def forward(self, x: torch.Tensor, ctx: StepContext, cache: PagedKV) -> torch.Tensor:
         k = self.kernels
         T = x.shape[0]
@@ -182,14 +219,16 @@ class Attention(Mixer):
         else:
             q = self._unfused(qkv, ctx, cache, tables)
         out = torch.empty_like(q)
-        if ctx.prefill_items.shape[0]:
-            k.paged_attention(q, cache.k, cache.v, tables.block_table, ctx.cu_q, ctx.k_len, ctx.prefill_items, mode=0,
-                              scale=self.scale, window=self.window, max_k_len=ctx.max_k_len, out=out)
-        if ctx.decode_items.shape[0]:
-            nseg = -(-ctx.max_decode_k_len // SEGMENT_KEYS)
-            scratch = ctx.attn_scratch(k.attn_scratch_floats(T, nq, d, nseg))
-            k.paged_attention(q, cache.k, cache.v, tables.block_table, ctx.cu_q, ctx.k_len, ctx.decode_items, mode=1,
-                              scale=self.scale, window=self.window, max_k_len=ctx.max_decode_k_len, nseg=nseg,
+        m = self._items(ctx.host)
+        prefill_items, decode_items = ctx.inputs["attention.prefill_items"], ctx.inputs["attention.decode_items"]
+        if prefill_items.shape[0]:
+            k.paged_attention(q, cache.k, cache.v, tables.block_table, ctx.cu_q, ctx.k_len, prefill_items, mode=0,
+                              scale=self.scale, window=self.window, max_k_len=ctx.host.k_len_bound, out=out)
+        if decode_items.shape[0]:
+            nseg = m["nseg"]
+            scratch = ctx.workspace(k.attn_scratch_floats(decode_items.shape[0], nq, d, nseg))
+            k.paged_attention(q, cache.k, cache.v, tables.block_table, ctx.cu_q, ctx.k_len, decode_items, mode=1,
+                              scale=self.scale, window=self.window, max_k_len=m["decode_bound"], nseg=nseg,
                               scratch=scratch, out=out)
         return k.gemm(out.view(T, nq * d), self.w_o)
 
@@ -277,20 +316,21 @@ class PreNormBlock(Block):
 
 @register_part("head", "linear_head")
 class LinearHead(Head):
-    """logits = x W^T without bias; W is the embedding table when tied
-    (src/exec/dense_swiglu_model.rs:976-984, qwen3/physical.py:131-134)."""
+    """logits = x W^T without bias (src/exec/dense_swiglu_model.rs:976-984).  A head tied to the embedding
+    is this same part: the architecture gives its weight the embedding table's tensor name, and the model
+    hands both parts the one tensor (python/vosti_kernels/model_families/qwen3/physical.py:131-134).
+    ``tied`` only records that for readers of the specification."""
 
-    def __init__(self, kernels: Kernels, vocab_size: int, hidden_size: int, tied: bool):
+    def __init__(self, kernels: Kernels, vocab_size: int, hidden_size: int, tied: bool = False):
         super().__init__(kernels)
-        self.vocab_size, self.hidden_size, self.tied = vocab_size, hidden_size, tied
+        self.vocab_size, self.hidden_size, self.tied = vocab_size, hidden_size, bool(tied)
         self.weight: torch.Tensor | None = None
 
     def params(self):
-        return {} if self.tied else {"weight": ParamSpec((self.vocab_size, self.hidden_size))}
+        return {"weight": ParamSpec((self.vocab_size, self.hidden_size))}
 
     def load(self, tensors):
-        if not self.tied:
-            self.weight = tensors["weight"]
+        self.weight = tensors["weight"]
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return self.kernels.gemm(x, self.weight)

@@ -75,14 +75,12 @@ def open_checkpoint(model_dir) -> Checkpoint:
 def check_against(model, ckpt: Checkpoint) -> None:
     """Raises one WeightError listing missing, unexpected and misshapen tensors."""
     expected = model.expected_tensors()
-    ignorable = set()
-    if getattr(model.head, "tied", False):
-        # A tied head has no tensor of its own; a file that stores one anyway is tolerated.
-        ignorable.add(model.spec.names.get("head.weight"))
+    ignorable = set(model.spec.ignored_names)
     missing = sorted(n for n in expected if n not in ckpt.entries)
     unexpected = sorted(n for n in ckpt.entries if n not in expected and n not in ignorable)
     wrong = []
-    for n, (_, _, ps) in expected.items():
+    for n, e in expected.items():
+        ps = e.spec
         if n in ckpt.entries:
             _, shape, dt = ckpt.entries[n]
             if tuple(shape) != tuple(ps.shape):
@@ -116,7 +114,7 @@ def load_weights(model, model_dir, device: str = "cuda") -> None:
     dtype = model.kernels.dtype
     tensors = {}
     # One tensor at a time: the whole checkpoint never sits in host memory.
-    for name, (_, _, ps) in expected.items():
+    for name, e in expected.items():
         t = ckpt.read([name])[name]
-        tensors[name] = convert(t, dtype, ps.keep_f32).contiguous().to(device)
+        tensors[name] = convert(t, dtype, e.spec.keep_f32).contiguous().to(device)
     model.load_tensors(tensors)

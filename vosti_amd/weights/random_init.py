@@ -67,7 +67,7 @@ def expected_tensor_specs(config) -> dict[str, tuple[tuple[int, ...], tuple]]:
     """Tensor name -> (shape, init) for a configuration; needs no GPU."""
     from ..models.decoder import DecoderModel
     model = DecoderModel(config.model_spec(), None)
-    return {name: (ps.shape, ps.init) for name, (_, _, ps) in model.expected_tensors().items()}
+    return {name: (e.spec.shape, e.spec.init) for name, e in model.expected_tensors().items()}
 
 
 def write_random_model(config, seed: int, out_dir: str | Path, dtype: torch.dtype = torch.bfloat16) -> Path:
@@ -89,7 +89,8 @@ def random_weights_on_gpu(model, seed: int) -> None:
     """Fills a model with the same values ``write_random_model`` would store in its compute type, on the GPU."""
     k = model.kernels
     tensors = {}
-    for name, (_, _, ps) in model.expected_tensors().items():
+    for name, e in model.expected_tensors().items():
+        ps = e.spec
         t = torch.empty(ps.shape, dtype=k.dtype, device="cuda")
         kind, p0, p1 = _init_params(ps.init)
         k.fill_random(t, tensor_seed(seed, name), kind, p0, p1)
