@@ -11,6 +11,9 @@
 // and the owner of the target walks its range again.  The result is a function
 // of the row, the temperature and the uniform number only.
 #include "common.h"
+#include "sampling.h"
+
+#include <mutex>
 
 #define SAMPLE_BLOCKS 32
 #define PARTIAL_THREADS 256
@@ -140,6 +143,61 @@ int vk_sample(int32_t* out, const elem_t* logits, const float* temps, const floa
   if (vk_check_launch("sample (partial)")) return 1;
   sample_final_kernel<<<R, FINAL_THREADS, 0, st>>>(out, pval, pidx, logits, temps, uniforms, V, row_stride);
   return vk_check_launch("sample");
+}
+
+}  // extern "C"
+
+// ---- the variant that allocates nothing (see sampling.h) ----
+// The partial maxima of vk_sample's first kernel, for up to VK_SAMPLE_STATIC_MAX_ROWS rows, in device
+// memory that belongs to the library: 8 bytes per (row, range).  Every GPU that the library runs on
+// holds its own copy of this array at its own address, until the process ends.
+static __device__ __align__(256) unsigned char scratch[(size_t)VK_SAMPLE_STATIC_MAX_ROWS * SAMPLE_BLOCKS * 8];
+
+#define VK_MAX_DEVICES 64
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[VK_MAX_DEVICES];      // device address of `scratch`, per device; null until asked for
+
+// The device address of `scratch` on the current device.  In host code the array's name is only a
+// handle for the runtime, not an address a kernel can use: the address is asked for once per device.
+static int static_scratch(void** ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return vk_fail("sample_static: hipGetDevice failed: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= VK_MAX_DEVICES) return vk_fail("sample_static: device index %d is beyond %d", dev, VK_MAX_DEVICES);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr)
+      return vk_fail("sample_static: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+    g_scratch_ptr[dev] = p;
+  }
+  *ptr = g_scratch_ptr[dev];
+  return 0;
+}
+
+extern "C" {
+
+int vk_sample_static_max_rows(void) { return VK_SAMPLE_STATIC_MAX_ROWS; }
+
+int vk_sample_static(int32_t* out, const elem_t* logits, const float* temps, const float* uniforms, int R, int V,
+                     int64_t row_stride, hipStream_t st) {
+  VK_REQUIRE(R >= 0 && V > 0, "sample_static: bad sizes R=%d V=%d", R, V);
+  VK_REQUIRE(R <= VK_SAMPLE_STATIC_MAX_ROWS, "sample_static: %d rows are more than the %d that the library's own scratch holds",
+             R, VK_SAMPLE_STATIC_MAX_ROWS);
+  VK_REQUIRE(row_stride >= V, "sample_static: row stride %lld smaller than V=%d", (long long)row_stride, V);
+  VK_REQUIRE(temps == nullptr || uniforms != nullptr, "sample_static: temperatures need uniform numbers");
+  VK_REQUIRE(out != nullptr && logits != nullptr, "sample_static: out and logits are needed");
+  if (R == 0) return 0;
+  void* base = nullptr;
+  if (static_scratch(&base)) return 1;
+  // Nothing has to start at zero: the first kernel writes every word that the second one reads.
+  float* pval = static_cast<float*>(base);
+  int* pidx = reinterpret_cast<int*>(pval + (size_t)VK_SAMPLE_STATIC_MAX_ROWS * SAMPLE_BLOCKS);
+  argmax_partial_kernel<<<dim3(R, SAMPLE_BLOCKS), PARTIAL_THREADS, 0, st>>>(pval, pidx, logits, V, row_stride);
+  if (vk_check_launch("sample_static (partial)")) return 1;
+  sample_final_kernel<<<R, FINAL_THREADS, 0, st>>>(out, pval, pidx, logits, temps, uniforms, V, row_stride);
+  return vk_check_launch("sample_static");
 }
 
 }  // extern "C"
