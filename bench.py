@@ -65,6 +65,7 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--graphs", type=int, default=1, choices=[0, 1], help="replay decode steps from captured HIP graphs")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill timing")
+    ap.add_argument("--no-per-kernel", action="store_true", help="skip the timing of the dominant kernels on their own")
     ap.add_argument("--prompt-tokens", type=int, default=PROMPT_TOKENS,
                     help="context length of the decode measurement (the prefill figure is always of 2,048 tokens)")
     ap.add_argument("--workload", default="decode8b", choices=["decode8b", "mixed14b", "prefix32b"])
@@ -101,7 +102,7 @@ def main() -> int:
     def prompt(n=None):
         return [rng.randrange(cfg.vocab_size) for _ in range(prompt_tokens if n is None else n)]
 
-    def decode_run(B: int, steps: int, warmup: int):
+    def decode_run(B: int, steps: int, warmup: int, per_kernel_into: dict | None = None):
         eng = Engine(model, num_pages=B * pages_per_request, page_size=page, max_num_seqs=B, max_num_batched_tokens=4096,
                      enable_prefix_cache=False, graphs=bool(args.graphs))
         sp = SamplingParams(max_tokens=GENERATED_TOKENS, ignore_eos=True)
@@ -118,6 +119,11 @@ def main() -> int:
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         ctx = prompt_tokens + warmup + 1 + (steps - 1) / 2.0          # mean keys per request over the timed steps
+        if per_kernel_into is not None:
+            try:
+                per_kernel_into["decode"] = kernel_times(model, cfg, eng.pool, B, int(ctx), elem, decode=True)
+            except Exception as e:      # the step's own figures stand without these
+                per_kernel_into["decode"] = {"error": f"{type(e).__name__}: {e}"}
         del eng
         torch.cuda.empty_cache()
         return dt / steps, ctx
@@ -137,7 +143,8 @@ def main() -> int:
             del eng
         return min(times[1:])
 
-    step_s, ctx = decode_run(args.batch, args.steps, args.warmup)
+    kernels: dict = {}
+    step_s, ctx = decode_run(args.batch, args.steps, args.warmup, None if args.no_per_kernel else kernels)
     value = args.batch / step_s
     bytes_step = decode_bytes(cfg, args.batch, ctx, elem)
     achieved = bytes_step / step_s / 1e9
@@ -165,8 +172,95 @@ def main() -> int:
             s, _ = decode_run(B, min(args.steps, 32), min(args.warmup, 4))
             points[name] = round(B / s, 2)
         record["points"] = points
+        if not args.no_per_kernel:
+            try:
+                from vosti_amd.cache import CachePool
+                pool = CachePool(model, page_size=page, num_pages=PROMPT_TOKENS // page, num_slots=1)
+                kernels["prefill"] = kernel_times(model, cfg, pool, PROMPT_TOKENS, PROMPT_TOKENS, elem, decode=False)
+            except Exception as e:
+                kernels["prefill"] = {"error": f"{type(e).__name__}: {e}"}
+    if kernels:
+        record["kernels"] = kernels
     print(json.dumps(record), flush=True)
     return 0
+
+
+def kernel_times(model, cfg, pool, M: int, keys: int, elem: int, decode: bool) -> dict:
+    """The dominant kernels on their own, at the step's shapes: each is recorded once per layer (with that
+    layer's weights and cache, so that nothing is warmer than in a step) into a graph, and the graph is
+    replayed.  decode: M rows of one token each over ``keys`` keys; else one prompt of M tokens.
+    Returns {kernel: {"us": per call, "GBps" or "TFLOPs": achieved, "frac": of the published peak}}."""
+    import torch
+    k = model.kernels
+    L = len(model.layers)
+    H, nq, nkv, d, I, V = (cfg.hidden_size, cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim,
+                           cfg.intermediate_size, cfg.vocab_size)
+    dt_name = "bf16" if elem == 2 else "fp32"
+    gen = torch.Generator(device="cuda").manual_seed(1)
+    rnd = lambda *shape: (torch.randn(*shape, generator=gen, device="cuda") * 0.5).to(k.dtype)
+    x, a, m, q = rnd(M, H), rnd(M, nq * d), rnd(M, I), rnd(M, nq, d)
+    P = pool.page_size
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device="cuda")
+    if decode:
+        W = -(-keys // P)
+        table = i32([[s * W + j for j in range(W)] for s in range(M)])
+        cu_q, k_len, items = i32(list(range(M + 1))), i32([keys] * M), i32([[s, 0] for s in range(M)])
+        nseg = -(-keys // 256)
+        scratch = torch.empty(k.attn_scratch_floats(M, nq, d, nseg), dtype=torch.float32, device="cuda")
+        attn = lambda c, out: k.paged_attention(q, c.k, c.v, table, cu_q, k_len, items, mode=1, scale=d ** -0.5,
+                                                max_k_len=keys, nseg=nseg, scratch=scratch, out=out)
+    else:
+        W = -(-M // P)
+        table = i32([list(range(W))])
+        cu_q, k_len = i32([0, M]), i32([M])
+        items = i32([[0, o] for o in range(0, M, 128)])
+        attn = lambda c, out: k.paged_attention(q, c.k, c.v, table, cu_q, k_len, items, mode=0, scale=d ** -0.5,
+                                                max_k_len=M, out=out)
+    layers = model.layers
+    o_qkv, o_h, o_i, o_attn = k.empty(M, (nq + 2 * nkv) * d), k.empty(M, H), k.empty(M, I), k.empty(M, nq, d)
+    head_rows = M if decode else 1
+    o_v = k.empty(head_rows, V)
+    work = {
+        "qkv": (lambda l: k.gemm(x, layers[l].mixer.w_qkv, out=o_qkv), (nq + 2 * nkv) * d * H, L),
+        "attention": (lambda l: attn(pool.entries[l], o_attn), None, L),
+        "o": (lambda l: k.gemm(a, layers[l].mixer.w_o, out=o_h), H * nq * d, L),
+        "gate_up": (lambda l: k.gemm_swiglu(x, layers[l].feed_forward.w_gate_up), 2 * I * H, L),
+        "down": (lambda l: k.gemm(m, layers[l].feed_forward.w_down, out=o_h), H * I, L),
+        "lm_head": (lambda l: k.gemm(x[:head_rows], model.head.weight, out=o_v), V * H, 1),
+    }
+    out = {}
+    reps = 5
+    for name, (fn, weight_elems, calls) in work.items():
+        for l in range(calls):                      # warm: every kernel variant is loaded before the capture
+            fn(l)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for l in range(calls):
+                fn(l)
+        graph.replay()
+        torch.cuda.synchronize()
+        t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0.record()
+        for _ in range(reps):
+            graph.replay()
+        t1.record()
+        torch.cuda.synchronize()
+        us = t0.elapsed_time(t1) * 1e3 / (reps * calls)
+        rows = head_rows if name == "lm_head" else M
+        if name == "attention":
+            flops = 4.0 * nq * d * (M * keys if decode else M * (M + 1) / 2)
+            nbytes = (M if decode else 1) * keys * 2 * nkv * d * elem
+        else:
+            flops, nbytes = 2.0 * rows * weight_elems, weight_elems * elem
+        if decode or name == "lm_head":      # one row through the head is a read of its weights, whatever the step
+            gbps = nbytes / us / 1e3
+            out[name] = {"us": round(us, 2), "GBps": round(gbps, 1), "frac": round(gbps / HBM_PEAK_GBS, 3)}
+        else:
+            tf = flops / us / 1e6
+            out[name] = {"us": round(us, 2), "TFLOPs": round(tf, 1), "frac": round(tf * 1e12 / PEAK_FLOPS[dt_name], 3)}
+        del graph
+    return out
 
 
 def progress(text: str, state={"t": 0.0}) -> None:

@@ -217,3 +217,15 @@ def test_no_page_lost_or_held_twice_under_random_orders(seed, prefix, windows):
     assert m.check() == ""
     assert all(m.available_pages(g) == 12 for g in range(len(windows)))
     assert m.free_slots() == 5
+
+
+def test_drop_cached_gives_every_unheld_page_back():
+    m = CacheManager(4, [GroupSpec(0, 8)], 4, True)
+    a, b = list(range(12)), list(range(100, 109))
+    m.add_request(1, a); feed(m, 1, a)
+    m.add_request(2, b); feed(m, 2, b); m.finish(2)             # two cached pages, one private tail freed
+    assert m.cached_blocks() == 2 and m.free_pages(0) == 8 - 3 - 2
+    assert m.drop_cached() == 2 and m.cached_blocks() == 0 and m.free_pages(0) == 5 and m.check() == ""
+    assert m.add_request(3, b) == 0                              # nothing left to reuse
+    m.finish(3); m.finish(1)
+    assert m.drop_cached() == 3 and m.free_pages(0) == 8 and m.check() == ""

@@ -187,3 +187,15 @@ def test_launcher_families_come_from_the_registry():
     class Probe:
         pass
     assert families()["probe_family"] == "ProbeForCausalLM"
+
+
+def test_multi_call_prompts_are_built_from_earlier_outputs():
+    # The reference's own vector: examples/support/engine_calls.rs:130-141.
+    from vosti_amd.launch import resolve_call_prompts
+    call = {"label": "reuse", "max_tokens": 2, "output_prefix_from": {"call": 0, "request": 0, "count": 2, "suffix": [8]}}
+    assert resolve_call_prompts(call, [([[1, 2]], [[3, 4, 5]])]) == [[1, 2, 3, 4, 8]]
+    with pytest.raises(SystemExit):
+        resolve_call_prompts(call, [])
+    with pytest.raises(SystemExit):
+        resolve_call_prompts(call, [([[1, 2]], [[3]])])
+    assert resolve_call_prompts({"prompts": [[1, 2], [3]]}, []) == [[1, 2], [3]]

@@ -220,6 +220,36 @@ def test_logits_digest(tiny_dirs, tmp_path, monkeypatch):
     assert [h for i, h in both if i == "1"] == [h for _, h in alone]
 
 
+def test_logits_observer_and_multi_call_driver(tiny_dirs, tmp_path):
+    """VOSTI_BENCH_CALLS: several calls through one engine, the second built from the first's output
+    (examples/support/engine_calls.rs); VOSTI_LOGITS_OBSERVER_DIR: every sampled row as a float32 .npy
+    with an index line that carries its hash, its step and the call it belongs to."""
+    import numpy as np
+    p = prompts("A", [20], seed=8)[0]
+    calls = {"prefix_caching": True, "calls": [
+        {"label": "first", "prompts": [p], "max_tokens": 3},
+        {"label": "second", "max_tokens": 2, "output_prefix_from": {"call": 0, "request": 0, "count": 2, "suffix": [7]}}]}
+    (tmp_path / "calls.json").write_text(json.dumps(calls))
+    env = dict(os.environ, MODEL_PATH=str(tiny_dirs["A"]), VOSTI_BENCH_CALLS=str(tmp_path / "calls.json"),
+               VOSTI_BENCH_CALL_RESULTS=str(tmp_path / "results.json"), VOSTI_LOGITS_OBSERVER_DIR=str(tmp_path / "obs"),
+               VOSTI_NUM_BLOCKS="8", VOSTI_PAGE_SIZE="16", VOSTI_DTYPE="float32", PYTHONPATH=str(ROOT))
+    r = subprocess.run([sys.executable, "-m", "vosti_amd.launch", "--kind", "engine", "--family", "qwen3"], env=env,
+                       capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0 and "CALLS_FINISHED 2" in r.stdout, r.stderr[-2000:]
+    rec = json.loads((tmp_path / "results.json").read_text())
+    first, second = rec
+    assert first["label"] == "first" and len(first["output_token_ids"][0]) == 3 and second["request_id_base"] == 1
+    assert second["input_token_ids"] == [p + first["output_token_ids"][0][:2] + [7]] and len(second["output_token_ids"][0]) == 2
+    index = [json.loads(l) for f in sorted((tmp_path / "obs").glob("observer-*.jsonl")) for l in f.read_text().splitlines()]
+    assert [r["phase"] for r in index] == ["call-0"] * 3 + ["call-1"] * 2
+    plain = PlainQwen3(tiny_dirs["A"], torch.float32)
+    for r, ids in zip(index, [p, p + first["output_token_ids"][0][:1], p + first["output_token_ids"][0][:2]]):
+        row = np.load(tmp_path / "obs" / r["artifact"])
+        assert row.dtype == np.float32 and row.shape == (256,) and r["argmax"] == int(row.argmax()) and r["finite"]
+        torch.testing.assert_close(torch.from_numpy(row), plain.logits(ids)[-1], rtol=1e-4, atol=2e-5)
+    assert index[0]["argmax"] == first["output_token_ids"][0][0]
+
+
 def test_smoke_entry():
     sys.path.insert(0, str(ROOT))
     import __graft_entry__

@@ -6,7 +6,7 @@ from ctypes import POINTER, c_char_p, c_int, c_int32, c_int64, c_uint64, c_void_
 
 from ..kernels import build
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 _LIB = None
 
 
@@ -35,7 +35,7 @@ def host_lib():
     sig("vh_cache_num_logical_pages", I, P, U, I)
     sig("vh_cache_available_pages", I, P, I)
     sig("vh_cache_free_pages", I, P, I)
-    for n in ("free_slots", "num_requests", "cached_blocks"):
+    for n in ("free_slots", "num_requests", "cached_blocks", "drop_cached"):
         sig(f"vh_cache_{n}", I, P)
     sig("vh_cache_prefix_hits", c_int64, P)
     sig("vh_cache_prefix_hit_requests", c_int64, P)

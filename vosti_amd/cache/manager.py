@@ -131,6 +131,10 @@ class CacheManager:
     def cached_blocks(self) -> int:
         return self._lib.vh_cache_cached_blocks(self._h)
 
+    def drop_cached(self) -> int:
+        """Gives every cached page that no request holds back to the free queue; returns how many."""
+        return self._lib.vh_cache_drop_cached(self._h)
+
     def prefix_hits(self) -> int:
         return self._lib.vh_cache_prefix_hits(self._h)
 

@@ -73,6 +73,12 @@ bool CacheManager::evict_one() {
   return false;
 }
 
+int CacheManager::drop_cached() {
+  int n = 0;
+  while (evict_one()) n += 1;
+  return n;
+}
+
 int CacheManager::available_pages(int g) const {
   return (int)groups_[g].free.size() + (prefix_cache_ ? (int)lru_.size() : 0);
 }

@@ -93,6 +93,10 @@ class CacheManager {
   int64_t prefix_hit_requests() const { return prefix_hit_requests_; }   // admissions that found a cached prefix
   int64_t evictions() const { return evictions_; }
   int cached_blocks() const { return (int)lru_.size(); }
+  // Gives every cached page (published, held by no request) back to the free queues; returns how many
+  // there were.  A caller that wants the next requests to find nothing to reuse calls it between them
+  // (the reference's reclaim_cached_leaves_until(capacity), examples/support/engine_calls.rs:72-82).
+  int drop_cached();
 
   // Empty string if every invariant holds, else a description of the first
   // violation: every page is free, cached or held, and never twice.

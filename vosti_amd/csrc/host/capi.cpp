@@ -20,7 +20,7 @@ struct SchedulerHandle {
 
 extern "C" {
 
-int vh_abi_version(void) { return 5; }
+int vh_abi_version(void) { return 6; }
 
 // ------------------------------------------------------------ cache manager
 void* vh_cache_create(int page_size, int n_groups, const int* windows, const int* num_pages, int num_slots,
@@ -54,6 +54,7 @@ int vh_cache_free_pages(void* h, int g) { return CM->free_pages(g); }
 int vh_cache_free_slots(void* h) { return CM->free_slots(); }
 int vh_cache_num_requests(void* h) { return CM->num_requests(); }
 int vh_cache_cached_blocks(void* h) { return CM->cached_blocks(); }
+int vh_cache_drop_cached(void* h) { return CM->drop_cached(); }
 int64_t vh_cache_prefix_hits(void* h) { return CM->prefix_hits(); }
 int64_t vh_cache_prefix_hit_requests(void* h) { return CM->prefix_hit_requests(); }
 int64_t vh_cache_evictions(void* h) { return CM->evictions(); }

@@ -9,9 +9,7 @@ to the host, where the scheduler appends them and retires finished requests.
 """
 from __future__ import annotations
 
-import hashlib
 import json
-import os
 from pathlib import Path
 
 import numpy as np
@@ -20,6 +18,7 @@ import torch
 from ..cache import CachePool
 from ..models import DecoderModel, load_model
 from ..sampling import SamplingParams, uniform_for
+from .observe import LogitsObserver
 from .scheduler import Scheduler
 from .step import ModelRunner, StepEntry
 
@@ -50,10 +49,9 @@ class Engine:
         self._next_id = 0
         self.steps = 0
         self.last_scheduled: list[int] = []
-        # VOSTI_LOGITS_DIGEST names a file: every sampled row's logits are hashed into it (as 32-bit
-        # floats, tagged with the row's index in the step), to compare runs that batch differently
-        # (python/vosti_kernels/kernels.py:1020-1033).
-        self.logits_digest_path = os.environ.get("VOSTI_LOGITS_DIGEST") or None
+        # VOSTI_LOGITS_DIGEST / VOSTI_LOGITS_OBSERVER_DIR: hashes or copies of every sampled logits row, to
+        # compare runs that batch differently (python/vosti_kernels/kernels.py:1020-1033).
+        self.observer = LogitsObserver()
 
     # ------------------------------------------------------------- requests
     def add_request(self, prompt_ids: list[int], params: SamplingParams | None = None, request_id: int | None = None) -> int:
@@ -104,11 +102,9 @@ class Engine:
         sampling = [r for r in rows if r.sample]
         logits = self.runner.run(entries)
         sampled: list[int] = []
-        if sampling and self.logits_digest_path:
-            data = self.kernels.to_f32(logits).cpu().numpy()
-            with open(self.logits_digest_path, "a") as f:
-                for i, r in enumerate(sampling):
-                    f.write(f"{rows.index(r)} {hashlib.sha256(data[i].tobytes()).hexdigest()}\n")
+        if sampling and self.observer.active:
+            self.observer.rows(self.kernels.to_f32(logits).cpu().numpy(), [rows.index(r) for r in sampling], self.steps,
+                               str(self.kernels.dtype))
         if sampling:
             temps = np.zeros(len(sampling), dtype=np.float32)
             unis = np.zeros(len(sampling), dtype=np.float32)

@@ -21,8 +21,11 @@ here; each also has a command-line option, which wins:
     VOSTI_OUTPUT_TOKENS        --output-tokens       write "index<TAB>ids" lines to this file
     VOSTI_BENCH_INPUT          --bench-input         TSV of MAX_TOKENS<TAB>IDS[<TAB>ARRIVAL_STEP] requests
     VOSTI_BENCH_WARMUP_INPUT   --bench-warmup-input  a TSV of other requests, served first by the same engine
+    VOSTI_BENCH_CALLS          --bench-calls         JSON of several calls served one after the other by one engine
+    VOSTI_BENCH_CALL_RESULTS   --bench-call-results  where their records go (a new JSON file)
     VOSTI_MAX_MODEL_LEN        --max-model-len       longest prompt plus output (default: the model's positions)
     VOSTI_LOGITS_DIGEST                              a file that gets "row sha256" for every sampled logits row
+    VOSTI_LOGITS_OBSERVER_DIR                        a folder that gets every sampled logits row as float32 .npy and an index
     VOSTI_ENGINE_STEP_TRACE    --step-trace          append one JSON line per step to this file
 
 Options without a counterpart in the reference: VOSTI_DTYPE / --dtype (bfloat16,
@@ -69,6 +72,8 @@ def engine_parser() -> argparse.ArgumentParser:
     p.add_argument("--output-tokens", default=_env("VOSTI_OUTPUT_TOKENS"))
     p.add_argument("--bench-input", default=_env("VOSTI_BENCH_INPUT"))
     p.add_argument("--bench-warmup-input", default=_env("VOSTI_BENCH_WARMUP_INPUT"))
+    p.add_argument("--bench-calls", default=_env("VOSTI_BENCH_CALLS"))
+    p.add_argument("--bench-call-results", default=_env("VOSTI_BENCH_CALL_RESULTS"))
     p.add_argument("--max-model-len", type=int, default=int(_env("VOSTI_MAX_MODEL_LEN", 0)))
     p.add_argument("--step-trace", default=_env("VOSTI_ENGINE_STEP_TRACE"))
     p.add_argument("--dtype", default=_env("VOSTI_DTYPE", "bfloat16"), choices=["bfloat16", "float32"])
@@ -105,6 +110,67 @@ def parse_prepared(path: str) -> list[tuple[int, list[int], int]]:
     return out
 
 
+def resolve_call_prompts(call: dict, prior: list[tuple[list[list[int]], list[list[int]]]]) -> list[list[int]]:
+    """The prompts of one call of a multi-call file: given outright, or built from an earlier call's
+    prompt, the first ``count`` tokens that call generated for it, and a suffix
+    (examples/support/engine_calls.rs:32-56)."""
+    src = call.get("output_prefix_from")
+    if src is None:
+        return [list(map(int, p)) for p in call.get("prompts", [])]
+    if not 0 <= src["call"] < len(prior):
+        raise SystemExit("bench calls: 'output_prefix_from' names a call that has not run yet")
+    prompts, outputs = prior[src["call"]]
+    if not 0 <= src["request"] < len(prompts):
+        raise SystemExit("bench calls: 'output_prefix_from' names a request that the call does not have")
+    out = outputs[src["request"]]
+    if src["count"] > len(out):
+        raise SystemExit("bench calls: 'output_prefix_from' wants more tokens than were generated")
+    return [prompts[src["request"]] + out[:src["count"]] + [int(t) for t in src.get("suffix", [])]]
+
+
+def run_calls(engine, path: str, results_path: str | None, eos, args) -> int:
+    """Several calls through one engine, one after the other (examples/support/engine_calls.rs:58-123):
+    {"prefix_caching": bool, "calls": [{"label", "prompts" | "output_prefix_from", "max_tokens"}]}.
+    Without prefix caching the cached pages are dropped before every call.  One record per call goes
+    to the results file, and ``CALLS_FINISHED <n>`` is printed."""
+    import torch
+    from .sampling import SamplingParams
+    spec = json.loads(Path(path).read_text())
+    calls = spec.get("calls") or []
+    if not calls:
+        raise SystemExit("bench calls: the file holds no calls")
+    if not results_path:
+        raise SystemExit("bench calls: VOSTI_BENCH_CALL_RESULTS (or --bench-call-results) is required")
+    if Path(results_path).exists():
+        raise SystemExit(f"bench calls: {results_path} exists already")
+    prior, records, base = [], [], 0
+    for index, call in enumerate(calls):
+        if engine.has_unfinished():
+            raise SystemExit("bench calls: the call before did not finish")
+        dropped = 0 if spec.get("prefix_caching") else engine.cache.drop_cached()
+        prompts = resolve_call_prompts(call, prior)
+        if not prompts or any(not p for p in prompts) or int(call.get("max_tokens", 0)) <= 0:
+            raise SystemExit("bench calls: a call has an empty prompt, an empty batch or no output budget")
+        os.environ["VOSTI_LOGITS_OBSERVER_PHASE"] = f"call-{index}"
+        params = SamplingParams(max_tokens=int(call["max_tokens"]), temperature=args.temperature, seed=args.seed,
+                                eos_token_ids=eos, ignore_eos=args.ignore_eos)
+        engine._next_id = max(engine._next_id, base)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        outputs = engine.generate(prompts, params)
+        wall = time.perf_counter() - t0
+        records.append({"label": call.get("label", str(index)), "request_id_base": base, "input_token_ids": prompts,
+                        "output_token_ids": outputs, "reclaimed_pages_before_call": dropped,
+                        "cache_isolated": not spec.get("prefix_caching"), "cache_page_tokens": engine.pool.page_size,
+                        "wall_s": wall, "graph_stats": dict(engine.runner.graph_stats)})
+        base += len(prompts)
+        prior.append((prompts, outputs))
+    with open(results_path, "x") as f:
+        json.dump(records, f)
+    print(f"CALLS_FINISHED {len(records)}")
+    return 0
+
+
 def eos_ids(model_path: str) -> tuple[int, ...]:
     path = Path(model_path) / "generation_config.json"
     if not path.is_file():
@@ -130,16 +196,20 @@ def run_engine(argv: list[str], family: str) -> int:
         raise SystemExit(f"{args.model_path} holds a {cfg.architecture}, not a {family} model")
     from .engine import Engine
     from .sampling import SamplingParams
-    if args.bench_input:
+    if args.bench_calls:
+        requests = []
+    elif args.bench_input:
         requests = parse_prepared(args.bench_input)
     else:
         requests = [(args.max_tokens, parse_ids(args.prompt_ids), 0)]
     warmup = parse_prepared(args.bench_warmup_input) if args.bench_input and args.bench_warmup_input else []
     eos = eos_ids(args.model_path)
     engine = Engine(args.model_path, dtype=args.dtype, num_pages=args.num_blocks, page_size=args.page_size,
-                    max_num_seqs=args.max_seqs or max(len(requests), len(warmup)),
+                    max_num_seqs=args.max_seqs or max(len(requests), len(warmup), 1 if not args.bench_calls else 8),
                     max_num_batched_tokens=args.max_batched_tokens, enable_prefix_cache=bool(args.prefix_cache),
                     max_model_len=args.max_model_len or None, graphs=bool(args.graphs))
+    if args.bench_calls:
+        return run_calls(engine, args.bench_calls, args.bench_call_results, eos, args)
     trace = open(args.step_trace, "a") if args.step_trace else None
     import torch
 
