@@ -39,7 +39,7 @@ HIPCC_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
 ]
-HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall", "-Wextra"]
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall", "-Wextra", "-ffp-contract=off"]
 
 
 def _writable_dir(preferred: Path, fallback_name: str) -> Path:
