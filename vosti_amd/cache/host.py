@@ -6,7 +6,7 @@ from ctypes import POINTER, c_char_p, c_int, c_int32, c_int64, c_uint64, c_void_
 
 from ..kernels import build
 
-ABI_VERSION = 6
+ABI_VERSION = 7
 _LIB = None
 
 
@@ -43,6 +43,8 @@ def host_lib():
     sig("vh_cache_fill_block_table", I, P, U, I, c_void_p, I)
     sig("vh_cache_fill_slots", I, P, U, I, I, I, c_void_p)
     sig("vh_cache_check", I, P, c_char_p, I)
+    sig("vh_cache_describe", I, P, I, c_void_p, c_void_p, c_void_p)
+    sig("vh_cache_fill_step", I, P, I, I, c_void_p, c_void_p, c_void_p, I, I, c_void_p, I, c_void_p)
     sig("vh_sched_create", P, P, I, I, I)
     sig("vh_sched_destroy", None, P)
     sig("vh_sched_add_request", I, P, U, PI, I, I, PI, I, I)

@@ -159,6 +159,29 @@ class CacheManager:
             self._raise(st, f"slots({rid}, group {group}, {start}..{start + n})")
         return out
 
+    def describe(self, rids: np.ndarray) -> tuple[np.ndarray, np.ndarray]:
+        """For the requests ``rids`` (uint64) in one call: [n, 3] = (committed length, pending tokens, state
+        slot) and [n, groups] = the block-table width each needs."""
+        n = rids.shape[0]
+        out = np.empty((n, 3), dtype=np.int32)
+        widths = np.empty((n, len(self.groups)), dtype=np.int32)
+        st = self._lib.vh_cache_describe(self._h, n, rids.ctypes.data, out.ctypes.data, widths.ctypes.data)
+        if st != OK:
+            self._raise(st, "describe")
+        return out, widths
+
+    def fill_step(self, group: int, rids: np.ndarray, starts: np.ndarray, n_tokens: np.ndarray, table: np.ndarray,
+                  slots: np.ndarray) -> None:
+        """Block table rows (``table`` [rows >= n, width]; the rest reads page 0) and the slots of every token
+        of the step (``slots`` [>= sum(n_tokens)]; the rest gets -1) of one group, in one call."""
+        n = rids.shape[0]
+        total = int(n_tokens.sum())
+        st = self._lib.vh_cache_fill_step(self._h, group, n, rids.ctypes.data, starts.ctypes.data, n_tokens.ctypes.data,
+                                          table.shape[0], table.shape[1], table.ctypes.data, slots.shape[0] - total,
+                                          slots.ctypes.data)
+        if st != OK:
+            self._raise(st, f"fill_step(group {group})")
+
     def check(self) -> str:
         """'' if every page and slot is accounted for exactly once, else the first violation."""
         buf = ctypes.create_string_buffer(512)

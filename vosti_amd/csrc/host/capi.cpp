@@ -20,7 +20,7 @@ struct SchedulerHandle {
 
 extern "C" {
 
-int vh_abi_version(void) { return 6; }
+int vh_abi_version(void) { return 7; }
 
 // ------------------------------------------------------------ cache manager
 void* vh_cache_create(int page_size, int n_groups, const int* windows, const int* num_pages, int num_slots,
@@ -63,6 +63,37 @@ int vh_cache_fill_block_table(void* h, uint64_t id, int g, int32_t* out, int wid
 }
 int vh_cache_fill_slots(void* h, uint64_t id, int g, int start, int n, int32_t* out) {
   return CM->fill_slots(id, g, start, n, out);
+}
+// What a step needs to know of its n requests, in one call: per request its committed length, its
+// pending tokens and its state slot (out: n x 3), and per request and group the block-table width it
+// needs (widths: n x n_groups).  Returns OK or the first request's error.
+int vh_cache_describe(void* h, int n, const uint64_t* ids, int32_t* out, int32_t* widths) {
+  const int G = CM->num_groups();
+  for (int i = 0; i < n; ++i) {
+    if (!CM->has_request(ids[i])) return UNKNOWN_REQUEST;
+    out[3 * i] = CM->length(ids[i]);
+    out[3 * i + 1] = CM->pending(ids[i]);
+    out[3 * i + 2] = CM->state_slot(ids[i]);
+    for (int g = 0; g < G; ++g) widths[i * G + g] = CM->num_logical_pages(ids[i], g);
+  }
+  return OK;
+}
+// The block table [rows, width] (rows beyond n, and entries beyond a request's pages, read page 0) and
+// the slots of every token of the step (n_tokens[i] tokens from starts[i] on; slots has room for their
+// sum plus `pad_tokens` entries, which get -1) of one group.
+int vh_cache_fill_step(void* h, int group, int n, const uint64_t* ids, const int32_t* starts, const int32_t* n_tokens,
+                       int rows, int width, int32_t* table, int pad_tokens, int32_t* slots) {
+  int64_t t = 0;
+  for (int i = 0; i < n; ++i) {
+    Status st = CM->fill_block_table(ids[i], group, table + (int64_t)i * width, width);
+    if (st != OK) return st;
+    st = CM->fill_slots(ids[i], group, starts[i], n_tokens[i], slots + t);
+    if (st != OK) return st;
+    t += n_tokens[i];
+  }
+  for (int64_t i = (int64_t)n * width; i < (int64_t)rows * width; ++i) table[i] = 0;
+  for (int i = 0; i < pad_tokens; ++i) slots[t + i] = -1;
+  return OK;
 }
 // Writes the first violated invariant into buf (empty if none); returns its length.
 int vh_cache_check(void* h, char* buf, int cap) {

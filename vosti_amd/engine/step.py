@@ -149,43 +149,56 @@ class ModelRunner:
         cache, spec = self.cache, self.model.spec
         real = len(entries)
         S = max(real, rows or 0)
-        q_lens = [len(e.tokens) for e in entries] + [1] * (S - real)
-        T = sum(q_lens)
-        starts = []
-        for e, n in zip(entries, q_lens):
-            if cache.pending(e.request_id) != n:
-                raise RuntimeError(f"request {e.request_id}: the cache holds pages for {cache.pending(e.request_id)} "
-                                   f"pending tokens, the step brings {n}")
-            starts.append(cache.length(e.request_id))
-        starts += [0] * (S - real)
-        ids = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries] + [np.zeros(S - real, dtype=np.int64)])
+        pad = S - real
+        rids = np.fromiter((e.request_id for e in entries), dtype=np.uint64, count=real)
+        n_tok = np.fromiter((len(e.tokens) for e in entries), dtype=np.int32, count=real)
+        info, needed = cache.describe(rids)              # one call for every request of the step
+        if not np.array_equal(info[:, 1], n_tok):
+            i = int(np.nonzero(info[:, 1] != n_tok)[0][0])
+            raise RuntimeError(f"request {entries[i].request_id}: the cache holds pages for {int(info[i, 1])} "
+                               f"pending tokens, the step brings {int(n_tok[i])}")
+        starts_a = np.ascontiguousarray(info[:, 0])
+        q_lens = n_tok.tolist() + [1] * pad
+        starts = starts_a.tolist() + [0] * pad
+        T = int(n_tok.sum()) + pad
+        if T == S:                                       # one token each: no concatenation of lists
+            ids = np.fromiter((e.tokens[0] for e in entries), dtype=np.int64, count=real)
+            positions = starts_a.astype(np.int32)
+        else:
+            ids = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries])
+            positions = np.concatenate([np.arange(s, s + n, dtype=np.int32) for s, n in zip(starts, q_lens[:real])])
         if ids.min() < 0 or ids.max() >= spec.vocab_size:
             raise ValueError(f"token id out of range [0, {spec.vocab_size})")
-        k_lens = [s + n for s, n in zip(starts, q_lens)]
-        if max(k_lens) > spec.max_positions:
-            raise ValueError(f"a request would reach {max(k_lens)} tokens; the model's positions end at {spec.max_positions}")
-        positions = np.concatenate([np.arange(s, s + n, dtype=np.int32) for s, n in zip(starts, q_lens)])
+        if pad:
+            ids = np.concatenate([ids, np.zeros(pad, dtype=np.int64)])
+            positions = np.concatenate([positions, np.zeros(pad, dtype=np.int32)])
+        k_lens_a = np.concatenate([starts_a + n_tok, np.ones(pad, dtype=np.int32)]) if pad else starts_a + n_tok
+        k_lens = k_lens_a.tolist()
+        if int(k_lens_a.max()) > spec.max_positions:
+            raise ValueError(f"a request would reach {int(k_lens_a.max())} tokens; the model's positions end at {spec.max_positions}")
         cu_q = np.zeros(S + 1, dtype=np.int32)
         np.cumsum(q_lens, out=cu_q[1:])
-        state_slots = [cache.state_slot(e.request_id) for e in entries] + [0] * (S - real)
-        want = []
-        for e, base, n in zip(entries, cu_q[:-1], q_lens):
-            for w in e.want:
-                if not 0 <= w < n:
-                    raise ValueError(f"request {e.request_id}: wanted place {w} is outside its {n} tokens")
-                want.append(int(base) + w)
-        want += [int(cu_q[s]) for s in range(real, S)]
+        state_slots = info[:, 2].tolist() + [0] * pad
+        if all(e.want == [0] for e in entries) and T == S:
+            want = cu_q[:-1].copy()
+        else:
+            want = []
+            for e, base, n in zip(entries, cu_q[:-1], q_lens):
+                for w in e.want:
+                    if not 0 <= w < n:
+                        raise ValueError(f"request {e.request_id}: wanted place {w} is outside its {n} tokens")
+                    want.append(int(base) + w)
+            want += [int(cu_q[s]) for s in range(real, S)]
+            want = np.asarray(want, dtype=np.int32)
         host = HostStep(q_lens=q_lens, starts=starts, k_lens=k_lens, state_slots=state_slots,
                         k_len_bound=bound if bound is not None else max(k_lens), frozen=bound is not None)
-        parts: list[np.ndarray] = [ids.astype(np.int32), positions, cu_q, np.asarray(k_lens, dtype=np.int32),
-                                   np.asarray(state_slots, dtype=np.int32), np.asarray(want, dtype=np.int32)]
+        parts: list[np.ndarray] = [ids.astype(np.int32), positions, cu_q, k_lens_a.astype(np.int32, copy=False),
+                                   np.asarray(state_slots, dtype=np.int32), want]
         for g in range(len(self.pool.group_windows)):
-            width = widths[g] if widths else self.needed_width(entries, g)
-            table = np.zeros((S, width), dtype=np.int32)
-            slots = np.full(T, -1, dtype=np.int32)
-            for s, e in enumerate(entries):
-                cache.block_table_row(e.request_id, g, width, table[s])
-                cache.slots(e.request_id, g, starts[s], q_lens[s], slots[cu_q[s]:cu_q[s + 1]])
+            width = widths[g] if widths else max(1, int(needed[:, g].max()))
+            table = np.empty((S, width), dtype=np.int32)
+            slots = np.empty(T, dtype=np.int32)
+            cache.fill_step(g, rids, starts_a, n_tok, table, slots)
             parts += [slots, table]
         names: list[str] = []
         for provider in self._providers.values():
@@ -202,7 +215,12 @@ class ModelRunner:
         return _Layout(parts, names, offsets, max(total, 4), host)
 
     def needed_width(self, entries: list[StepEntry], group: int) -> int:
-        return max(1, max(self.cache.num_logical_pages(e.request_id, group) for e in entries))
+        return self.needed_widths(entries)[group]
+
+    def needed_widths(self, entries: list[StepEntry]) -> list[int]:
+        """The block-table width that the step's requests need, per group."""
+        rids = np.fromiter((e.request_id for e in entries), dtype=np.uint64, count=len(entries))
+        return [max(1, int(w)) for w in self.cache.describe(rids)[1].max(axis=0)]
 
     def _context(self, lay: _Layout, dev: torch.Tensor):
         views = [dev[o:o + p.size].view(p.shape) for p, o in zip(lay.parts, lay.offsets)]
@@ -239,7 +257,7 @@ class ModelRunner:
         if self._poisoned is not None:
             raise GraphError(f"graph replay is switched off after a failure: {self._poisoned}")
         P = self.pool.page_size
-        widths = [width_bucket(self.needed_width(entries, g)) for g in range(len(self.pool.group_windows))]
+        widths = [width_bucket(w) for w in self.needed_widths(entries)]
         # A mixer with state of its own would have to be told which rows are padding: no padding then.
         rows = len(entries) if self.pool.has_state else next((b for b in ROW_BUCKETS if b >= len(entries)), len(entries))
         key = (rows, tuple(widths))

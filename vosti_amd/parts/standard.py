@@ -169,33 +169,32 @@ class Attention(Mixer):
     def _items(step: HostStep) -> dict:
         m = step.memo.get("attention.items")
         if m is None:
-            prefill, decode, decode_keys = [], [], 0
-            for s, n in enumerate(step.q_lens):
-                if n == 1:
-                    decode.append((s, 0))
-                    decode_keys = max(decode_keys, step.k_lens[s])
-                else:
-                    prefill.extend((s, off) for off in range(0, n, ATTN_ITEM_ROWS))
+            q = np.asarray(step.q_lens, dtype=np.int32)
+            single = q == 1
+            seqs = np.nonzero(single)[0].astype(np.int32)
+            decode = np.stack([seqs, np.zeros_like(seqs)], axis=1) if seqs.size else np.zeros((0, 2), dtype=np.int32)
+            prefill = [(s, off) for s in np.nonzero(~single)[0].tolist() for off in range(0, int(q[s]), ATTN_ITEM_ROWS)]
+            decode_keys = int(np.asarray(step.k_lens, dtype=np.int32)[single].max()) if seqs.size else 0
             # Recorded launches must cover every length that the tables can hold.
             bound = step.k_len_bound if step.frozen else decode_keys
-            m = {"prefill": prefill, "decode": decode, "decode_bound": bound, "nseg": -(-bound // SEGMENT_KEYS)}
+            m = {"prefill": np.asarray(prefill, dtype=np.int32).reshape(-1, 2), "decode": decode, "decode_bound": bound,
+                 "nseg": -(-bound // SEGMENT_KEYS)}
             step.memo["attention.items"] = m
         return m
 
     @classmethod
     def _items_arrays(cls, step: HostStep) -> dict:
         m = cls._items(step)
-        return {"attention.prefill_items": np.asarray(m["prefill"], dtype=np.int32).reshape(-1, 2),
-                "attention.decode_items": np.asarray(m["decode"], dtype=np.int32).reshape(-1, 2)}
+        return {"attention.prefill_items": m["prefill"], "attention.decode_items": m["decode"]}
 
     def step_inputs(self, step: HostStep):
         return self._items_arrays(step)
 
     def workspace_floats(self, step: HostStep) -> int:
         m = self._items(step)
-        if not m["decode"]:
+        if not m["decode"].shape[0]:
             return 0
-        return self.kernels.attn_scratch_floats(len(m["decode"]), self.nq, self.d, m["nseg"])
+        return self.kernels.attn_scratch_floats(m["decode"].shape[0], self.nq, self.d, m["nseg"])
 
     def forward(self, x: torch.Tensor, ctx: StepContext, cache: PagedKV) -> torch.Tensor:
         k = self.kernels
