@@ -1,0 +1,149 @@
+"""The native engine (vosti_engine) against the Python engine and the plain implementation.
+
+Both engines drive the same kernels, cache manager and scheduler; what differs is everything between:
+configuration, weight loading, parts, step layout, graph replay, sampling state.  So the native engine's
+tokens must be the Python engine's, token for token, and pass the same checks against the plain
+implementation.  (The two compute the rotary frequencies with different pow routines, which may differ
+in the last bit of a frequency; the checks against the plain implementation hold for each alone.)"""
+import json
+import os
+import shutil
+import subprocess
+
+import pytest
+import torch
+from safetensors.torch import load_file, save_file
+
+from conftest import TINY
+from plain_qwen3 import PlainQwen3
+from test_engine_gpu import DTYPES, check_greedy_against_plain, engine, prompts
+from vosti_amd.kernels import build
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def program():
+    return str(build.ensure("engine", verbose=False))
+
+
+def run_native(program, dtype_name, env=None, args=(), expect=0):
+    lib = build.ensure({"float32": "f32", "bfloat16": "bf16"}[dtype_name], verbose=False)
+    base = {k: v for k, v in os.environ.items() if not k.startswith("VOSTI_") and k != "MODEL_PATH"}
+    r = subprocess.run([program, "--family", "qwen3", "--dtype", dtype_name, "--lib-dir", str(lib.parent), *args],
+                       env=dict(base, **(env or {})), capture_output=True, text=True, timeout=110)
+    assert r.returncode == expect, (r.returncode, r.stderr[-2000:])
+    return r
+
+
+def tsv(path, requests):
+    path.write_text("".join(f"{m}\t{','.join(map(str, ids))}\t{a}\n" for m, ids, a in requests))
+
+
+def read_outputs(path):
+    return [[int(t) for t in line.split("\t")[1].split(",")] for line in path.read_text().splitlines()]
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_one_prompt_through_the_environment(program, tiny_dirs, tmp_path, name, dtype_name):
+    """The reference's way of calling its engine example: everything through environment variables."""
+    from vosti_amd.sampling import SamplingParams
+    p = prompts(name, [37], seed=5)[0]
+    page = TINY[name][1]
+    env = dict(MODEL_PATH=str(tiny_dirs[name]), VOSTI_PROMPT_IDS=",".join(map(str, p)), VOSTI_MAX_TOKENS="12",
+               VOSTI_NUM_BLOCKS="6", VOSTI_PAGE_SIZE=str(page), VOSTI_OUTPUT_TOKENS=str(tmp_path / "out.tsv"),
+               VOSTI_ENGINE_STEP_TRACE=str(tmp_path / "trace.jsonl"))
+    r = run_native(program, dtype_name, env)
+    line = [l for l in r.stdout.splitlines() if l.startswith("MODEL_OUTPUT_TOKEN_IDS=")][0]
+    out = json.loads(line.split("=", 1)[1])
+    assert len(out) == 12
+    check_greedy_against_plain(PlainQwen3(tiny_dirs[name], DTYPES[dtype_name]), p, out, dtype_name,
+                               PlainQwen3(tiny_dirs[name], torch.float32))
+    assert read_outputs(tmp_path / "out.tsv") == [out]
+    # The Python engine, told the same: the same tokens and the same step trace.
+    trace = tmp_path / "py.jsonl"
+    with open(trace, "w") as f:
+        py = engine(tiny_dirs[name], dtype_name, num_pages=6, page_size=page, max_num_seqs=1).generate(
+            [p], SamplingParams(max_tokens=12), trace=f)
+    assert py == [out]
+    assert [json.loads(l) for l in (tmp_path / "trace.jsonl").read_text().splitlines()] == [json.loads(l) for l in trace.read_text().splitlines()]
+
+
+@pytest.mark.parametrize("graphs", [0, 1])
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_staggered_workload_with_temperature(program, tiny_dirs, tmp_path, dtype_name, graphs):
+    """Six requests with prompts of 2 to 120 tokens that arrive at different steps, temperature 0.8 with a
+    seed each, three rows a step, 48 tokens a step and few pages: prompts are cut into portions, requests
+    wait, pages are used again, and (graphs 1) decode steps are replayed from recordings with padding rows.
+    Tokens, cache statistics and graph counts are the Python engine's under the same settings."""
+    from vosti_amd.sampling import SamplingParams
+    ps = prompts("B", [2, 120, 31, 64, 9, 77])
+    arrivals = [0, 0, 2, 4, 8, 12]
+    tsv(tmp_path / "reqs.tsv", [(24, p, a) for p, a in zip(ps, arrivals)])
+    r = run_native(program, dtype_name, args=["--model-path", str(tiny_dirs["B"]), "--bench-input", str(tmp_path / "reqs.tsv"),
+                                              "--output-tokens", str(tmp_path / "out.tsv"), "--num-blocks", "40", "--page-size", "8",
+                                              "--max-seqs", "3", "--max-batched-tokens", "48", "--temperature", "0.8", "--seed", "100",
+                                              "--graphs", str(graphs)])
+    outs = read_outputs(tmp_path / "out.tsv")
+    assert [len(o) for o in outs] == [24] * 6
+    e = engine(tiny_dirs["B"], dtype_name, num_pages=40, page_size=8, max_num_seqs=3, max_num_batched_tokens=48, graphs=bool(graphs))
+    params = [SamplingParams(max_tokens=24, temperature=0.8, seed=100 + i) for i in range(6)]
+    assert e.generate(ps, params, arrival_steps=arrivals) == outs
+    assert f"BENCH batch=6 prompt_tokens={sum(map(len, ps))} output_tokens=144" in r.stdout
+    stats = json.loads([l for l in r.stdout.splitlines() if l.startswith("CACHE_STATS ")][0].split(" ", 1)[1])
+    assert stats == {"admitted_requests": 6, "requests_with_reuse": e.cache.prefix_hit_requests(),
+                     "reused_prefix_blocks": e.cache.prefix_hits(), "preemptions": e.scheduler.preemptions()}
+    if graphs:
+        g = json.loads([l for l in r.stdout.splitlines() if l.startswith("GRAPH_STATS ")][0].split(" ", 1)[1])
+        assert g == e.runner.graph_stats and g["captured"] >= 2 and g["replayed"] > g["captured"]
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_shared_prefixes_end_tokens_and_stored_types(program, tiny_dirs, tmp_path, dtype_name):
+    """A folder whose tensors are stored in the other float type than the one computed in (so every tensor
+    is converted while loading), with end tokens in generation_config.json; requests that share a prefix
+    find each other's pages."""
+    from vosti_amd.sampling import SamplingParams
+    d = tmp_path / "model"
+    shutil.copytree(tiny_dirs["A"], d)
+    stored = torch.float32 if dtype_name == "bfloat16" else torch.bfloat16
+    t = load_file(str(d / "model.safetensors"))
+    save_file({n: (v.to(stored) if n != "model.norm.weight" else v.float()) for n, v in t.items()}, str(d / "model.safetensors"))
+    shared = prompts("A", [40], seed=9)[0]
+    ps = [shared + [5], shared + [9, 11], shared[:20] + [3]]
+    free = engine(d, dtype_name, num_pages=16, page_size=16, max_num_seqs=3).generate(ps, SamplingParams(max_tokens=10))
+    eos = sorted({free[0][4], free[1][6]})            # tokens that requests 0 and 1 emit on their way
+    (d / "generation_config.json").write_text(json.dumps({"eos_token_id": eos}))
+    tsv(tmp_path / "reqs.tsv", [(10, p, a) for p, a in zip(ps, [0, 3, 3])])
+    r = run_native(program, dtype_name, args=["--model-path", str(d), "--bench-input", str(tmp_path / "reqs.tsv"), "--num-blocks", "16",
+                                              "--page-size", "16", "--output-tokens", str(tmp_path / "out.tsv")])
+    outs = read_outputs(tmp_path / "out.tsv")
+    e = engine(d, dtype_name, num_pages=16, page_size=16, max_num_seqs=3)
+    py = e.generate(ps, SamplingParams(max_tokens=10, eos_token_ids=tuple(eos)), arrival_steps=[0, 3, 3])
+    assert outs == py and len(outs[0]) < 10 and outs[0][-1] in eos
+    assert f'"requests_with_reuse":{e.cache.prefix_hit_requests()},"reused_prefix_blocks":{e.cache.prefix_hits()}' in r.stdout
+    assert e.cache.prefix_hits() >= 3
+    # --ignore-eos: to the end of the budget again.
+    run_native(program, dtype_name, args=["--model-path", str(d), "--bench-input", str(tmp_path / "reqs.tsv"), "--num-blocks", "16",
+                                          "--page-size", "16", "--output-tokens", str(tmp_path / "out2.tsv"), "--ignore-eos"])
+    assert read_outputs(tmp_path / "out2.tsv") == engine(d, dtype_name, num_pages=16, page_size=16, max_num_seqs=3).generate(
+        ps, SamplingParams(max_tokens=10, eos_token_ids=tuple(eos), ignore_eos=True), arrival_steps=[0, 3, 3])
+
+
+def test_one_error_for_weights_that_do_not_fit(program, tiny_dirs, tmp_path):
+    d = tmp_path / "model"
+    shutil.copytree(tiny_dirs["B"], d)
+    t = load_file(str(d / "model.safetensors"))
+    del t["model.layers.1.mlp.up_proj.weight"]
+    t["model.layers.0.self_attn.q_norm.weight"] = torch.ones(8)
+    t["model.layers.7.extra"] = torch.zeros(2)
+    save_file(t, str(d / "model.safetensors"))
+    r = run_native(program, "bfloat16", args=["--model-path", str(d)], expect=1)
+    assert "missing (1): model.layers.1.mlp.up_proj.weight" in r.stderr
+    assert "unexpected (1): model.layers.7.extra" in r.stderr
+    assert "wrong shape or type (1): model.layers.0.self_attn.q_norm.weight: file has [8], model needs [32]" in r.stderr
+    # Pages that cannot hold the request: refused, not run.
+    r = run_native(program, "bfloat16", args=["--model-path", str(tiny_dirs["B"]), "--prompt-ids", ",".join(["7"] * 100),
+                                              "--num-blocks", "2", "--page-size", "8"], expect=1)
+    assert "more cache pages than the pool has" in r.stderr

@@ -1,10 +1,13 @@
 """Compiles the native libraries in-tree.
 
-Three shared libraries are built from ``vosti_amd/csrc``:
+Three shared libraries and one program are built from ``vosti_amd/csrc``:
 
 * ``libvosti_bf16.so`` and ``libvosti_f32.so``: the gfx950 kernels, the same
   sources compiled with ``-DVK_BF16`` or ``-DVK_F32`` (hipcc);
-* ``libvosti_host.so``: the cache manager and the scheduler (g++, no GPU code).
+* ``libvosti_host.so``: the cache manager and the scheduler (g++, no GPU code);
+* ``vosti_engine``: the native engine and its command line (``csrc/engine`` with
+  the cache manager and the scheduler compiled in; g++ against the HIP runtime;
+  it loads the kernel library of the chosen precision from its own folder).
 
 A library is rebuilt when the hash of its sources, headers and flags differs
 from the one recorded beside it.  ``ensure()``
@@ -63,24 +66,45 @@ def build_dir() -> Path:
     return _writable_dir(PACKAGE_DIR.parent / "_build", "build")
 
 
+def _file_name(name: str) -> str:
+    return "vosti_engine" if name == "engine" else f"libvosti_{name}.so"
+
+
 def lib_path(name: str) -> Path:
-    """Path of a built library: the in-tree one if present, else the fallback location."""
-    in_tree = PACKAGE_DIR / "_lib" / f"libvosti_{name}.so"
+    """Path of a built library or program: the in-tree one if present, else the fallback location."""
+    in_tree = PACKAGE_DIR / "_lib" / _file_name(name)
     if in_tree.exists():
         return in_tree
-    return lib_dir() / f"libvosti_{name}.so"
+    return lib_dir() / _file_name(name)
+
+
+def rocm_root() -> Path:
+    return Path(os.environ.get("ROCM_PATH") or "/opt/rocm")
 
 
 def _sources(name: str) -> tuple[list[Path], list[Path]]:
+    host = CSRC / "host"
     if name == "host":
-        return sorted((CSRC / "host").glob("*.cpp")), sorted((CSRC / "host").glob("*.h"))
+        return sorted(host.glob("*.cpp")), sorted(host.glob("*.h"))
+    if name == "engine":
+        engine = CSRC / "engine"
+        return (sorted(engine.glob("*.cpp")) + [host / "cache_manager.cpp", host / "scheduler.cpp"],
+                sorted(engine.glob("*.h")) + sorted(host.glob("*.h")))
     return sorted(CSRC.glob("*.hip")), sorted(CSRC.glob("*.h"))
+
+
+def _flags(name: str) -> list[str]:
+    if name == "host":
+        return HOST_FLAGS
+    if name == "engine":
+        return HOST_FLAGS + ["-I", str(rocm_root() / "include")]
+    return HIPCC_FLAGS + [f"-D{GPU_LIBS[name]}"]
 
 
 def source_hash(name: str) -> str:
     srcs, hdrs = _sources(name)
     h = hashlib.sha256()
-    h.update(repr((HOST_FLAGS if name == "host" else HIPCC_FLAGS + [GPU_LIBS[name]])).encode())
+    h.update(repr(_flags(name)).encode())
     for p in srcs + hdrs:
         h.update(p.name.encode())
         h.update(p.read_bytes())
@@ -107,17 +131,17 @@ def _run(cmd: list[str], what: str) -> None:
 
 
 def build(name: str, verbose: bool = True) -> Path:
-    """Compile library ``name`` ('bf16', 'f32' or 'host') unconditionally."""
+    """Compile library ``name`` ('bf16', 'f32' or 'host') or the program 'engine' unconditionally."""
     srcs, _ = _sources(name)
     if not srcs:
         raise RuntimeError(f"no sources for library {name!r} under {CSRC}")
     obj_dir = build_dir() / name
     obj_dir.mkdir(parents=True, exist_ok=True)
-    if name == "host":
-        compiler, flags = _find("g++", "/usr/bin/g++"), HOST_FLAGS
+    if name in ("host", "engine"):
+        compiler = _find("g++", "/usr/bin/g++")
     else:
         compiler = _find("hipcc", "/opt/rocm/bin/hipcc")
-        flags = HIPCC_FLAGS + [f"-D{GPU_LIBS[name]}"]
+    flags = _flags(name)
     t0 = time.time()
 
     def compile_one(src: Path) -> Path:
@@ -130,7 +154,16 @@ def build(name: str, verbose: bool = True) -> Path:
     workers = max(1, min(len(srcs), int(os.environ.get("MAX_JOBS", os.cpu_count() or 4)), 16))
     with ThreadPoolExecutor(workers) as pool:
         objs = list(pool.map(compile_one, srcs))
-    out = lib_dir() / f"libvosti_{name}.so"
+    out = lib_dir() / _file_name(name)
+    if name == "engine":
+        tmp = out.with_name(f"{out.name}.tmp{os.getpid()}")
+        rocm_lib = str(rocm_root() / "lib")
+        _run([compiler, "-o", str(tmp), *map(str, objs), "-L", rocm_lib, "-lamdhip64", "-ldl", f"-Wl,-rpath,{rocm_lib}"], out.name)
+        os.replace(tmp, out)
+        Path(str(out) + ".srchash").write_text(source_hash(name) + "\n")
+        if verbose:
+            print(f"[vosti_amd build] {name}: linked {out} ({time.time() - t0:.0f}s)", file=sys.stderr, flush=True)
+        return out
     tmp = out.with_suffix(f".tmp{os.getpid()}.so")
     link = [compiler, "-shared", "-fPIC", "-o", str(tmp), *map(str, objs)]
     if name != "host":
@@ -160,7 +193,7 @@ def ensure(name: str, verbose: bool = True) -> Path:
 
 
 def build_all(verbose: bool = True) -> None:
-    for name in ("host", "bf16", "f32"):
+    for name in ("host", "engine", "bf16", "f32"):
         build(name, verbose)
 
 
