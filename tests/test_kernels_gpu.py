@@ -55,6 +55,14 @@ def test_gemm(dtype, M, N, K):
         for code in codes:
             got_s = k.gemm(a.cuda(), w.cuda(), kernel=code)
             assert torch.equal(got_s, got_t), f"the skinny kernel {code} and the tiled kernel must agree bitwise"
+        # The route through chunk sums in a workspace (17 to 64 rows of 16-bit elements, K in whole chunks).
+        need = k.gemm_workspace_floats(M, N, K, force=True)
+        assert (need > 0) == (M > 16 and K % 512 == 0 and dtype == torch.bfloat16)
+        if need:
+            ws = torch.full((need + 5,), float("nan"), device="cuda")       # what a call before may have left
+            assert torch.equal(k.gemm(a.cuda(), w.cuda(), kernel=14, workspace=ws), got_t), "chunk sums"
+            with pytest.raises(Exception, match="workspace"):
+                k.gemm(a.cuda(), w.cuda(), kernel=14, workspace=ws[:need - 1])
     # A row of a batch equals the same row alone, bitwise.
     for r in {0, M // 2, M - 1}:
         one = k.gemm(a[r:r + 1].cuda(), w.cuda())
@@ -72,10 +80,14 @@ def test_gemm_every_row_count(dtype, N, K):
     full = k.gemm(a, w, kernel=2)
     torch.testing.assert_close(full.float().cpu(), (a.double().cpu() @ w.double().cpu().t()).to(dtype).float(), **tol(dtype))
     fused = k.gemm_swiglu(a, w) if N % 2 == 0 else None
+    ws = torch.empty(1 << 24, device="cuda")      # enough for the route through chunk sums at every size here
     for M in list(range(1, 70)) + [95, 96, 97, 127, 128, 129, 191, 192, 193, 255, 256, 257, 300, 330]:
         assert torch.equal(k.gemm(a[:M], w), full[:M]), M
+        assert torch.equal(k.gemm(a[:M], w, workspace=ws), full[:M]), M       # the kernel chosen when there is a workspace
         if fused is not None:
             assert torch.equal(k.gemm_swiglu(a[:M], w), fused[:M]), M
+            if k.gemm_workspace_floats(M, N, K, swiglu=True, force=True):
+                assert torch.equal(k.gemm_swiglu(a[:M], w, workspace=ws, split=True), fused[:M]), M
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

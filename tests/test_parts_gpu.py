@@ -91,6 +91,37 @@ def test_embedding_norm_head_swiglu(dtype):
     torch.testing.assert_close(ffn.forward(x.cuda(), None).float().cpu(), ref, **tol(dtype))
 
 
+def test_projections_with_a_workspace_give_the_same_bits():
+    """With 17 to 64 rows the larger projections go through chunk sums in the step's workspace; the parts
+    announce how much of it they need, and the result is what they compute without one."""
+    from vosti_amd.kernels import kernels_for
+    from vosti_amd.parts import HostStep
+    dtype, k = torch.bfloat16, kernels_for(torch.bfloat16)
+    host = HostStep(q_lens=[40], starts=[0], k_lens=[40], state_slots=[0], k_len_bound=40)
+    ffn = build("feed_forward", "swiglu", dtype, hidden_size=1024, intermediate_size=8192)
+    load(ffn, dtype, scale=0.03)
+    assert ffn.workspace_floats(host) == k.gemm_workspace_floats(40, 1024, 8192) > 0
+    x = rand((40, 1024), dtype, 3).cuda()
+    ctx = step_context(k, [0], [40], 64, [[0]], 1)
+    ctx.workspace = lambda n, buf=torch.full((ffn.workspace_floats(host),), float("nan"), device="cuda"): buf
+    assert torch.equal(ffn.forward(x, ctx), ffn.forward(x, None))
+    rope = PartSpec("rotary", {"head_dim": 128, "rotary_dim": 128, "theta": 1e4, "max_positions": 64})
+    att = build("mixer", "attention", dtype, hidden_size=2048, num_heads=16, num_kv_heads=8, head_dim=128, scale=128 ** -0.5,
+                position=rope)
+    load(att, dtype, scale=0.03)
+    assert att.workspace_floats(host) == k.gemm_workspace_floats(40, 32 * 128, 2048) > 0
+    from vosti_amd.parts import PagedKV
+    x = rand((40, 2048), dtype, 4).cuda()
+    outs = []
+    for with_workspace in (True, False):
+        cache = PagedKV(torch.zeros(1, 8, 64, 128, dtype=dtype, device="cuda"), torch.zeros(1, 8, 128, 64, dtype=dtype, device="cuda"), 0, 64)
+        ctx = step_context(k, [0], [40], 64, [[0]], 1)
+        if not with_workspace:
+            ctx.workspace = None
+        outs.append(att.forward(x, ctx, cache))
+    assert torch.equal(outs[0], outs[1])
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_rotary_part(dtype):
     rot = build("position", "rotary", dtype, head_dim=32, rotary_dim=32, theta=1e4, max_positions=64)

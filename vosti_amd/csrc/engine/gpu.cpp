@@ -86,6 +86,9 @@ struct Kernels::Fn {
   int (*gemm)(P, CP, CP, int, int, int, int64_t, int64_t, int, hipStream_t);
   int (*gemm_swiglu)(P, CP, CP, int, int, int, int64_t, int64_t, hipStream_t);
   int (*gemm_swiglu_supported)(int, int, int);
+  int (*gemm_split)(P, CP, CP, int, int, int, int64_t, int64_t, int, P, int64_t, hipStream_t);
+  int64_t (*gemm_split_floats)(int, int, int, int);
+  int (*gemm_split_preferred)(int, int, int, int);
   int (*qkv_post)(CP, int64_t, P, P, P, CP, CP, int, CP, CP, int, CP, CP, int, int, int, int, int, float, hipStream_t);
   int (*paged_attention)(P, CP, CP, CP, CP, int, CP, CP, CP, int, int, int, P, int, int, int, int, int, int, float, hipStream_t);
   int (*sample)(P, CP, CP, CP, P, int, int, int64_t, hipStream_t);
@@ -95,7 +98,7 @@ struct Kernels::Fn {
   int (*attn_item_rows)();
 };
 
-static constexpr int KERNEL_ABI = 11;
+static constexpr int KERNEL_ABI = 12;
 
 Kernels::Kernels(const std::string& lib_dir, const std::string& name) : name_(name), fn_(new Fn) {
   if (name == "bf16") dtype_ = DType::BF16;
@@ -117,6 +120,7 @@ Kernels::Kernels(const std::string& lib_dir, const std::string& name) : name_(na
   VK(embedding, "vk_embedding"); VK(rmsnorm, "vk_rmsnorm"); VK(add_rmsnorm, "vk_add_rmsnorm"); VK(swiglu, "vk_swiglu");
   VK(gather_rows, "vk_gather_rows"); VK(cast_to_f32, "vk_cast_to_f32"); VK(rope_tables, "vk_rope_tables");
   VK(gemm, "vk_gemm"); VK(gemm_swiglu, "vk_gemm_swiglu"); VK(gemm_swiglu_supported, "vk_gemm_swiglu_supported");
+  VK(gemm_split, "vk_gemm_split"); VK(gemm_split_floats, "vk_gemm_split_floats"); VK(gemm_split_preferred, "vk_gemm_split_preferred");
   VK(qkv_post, "vk_qkv_post"); VK(paged_attention, "vk_paged_attention"); VK(sample, "vk_sample");
   VK(sample_scratch_words, "vk_sample_scratch_words"); VK(attn_scratch_floats, "vk_attn_scratch_floats");
   VK(attn_segment_keys, "vk_attn_segment_keys"); VK(attn_item_rows, "vk_attn_item_rows");
@@ -230,26 +234,44 @@ void Kernels::rope_tables(Tensor& cos, Tensor& sin, const Tensor& inv_freq) {
   call(fn_->rope_tables(cos.data, sin.data, inv_freq.data, (int)cos.dim(0), (int)half, stream));
 }
 
-Tensor Kernels::gemm(const Tensor& act, const Tensor& w) {
+int64_t Kernels::gemm_workspace_floats(int64_t M, int64_t rows, int64_t K, bool swiglu) const {
+  if (!fn_->gemm_split_preferred((int)M, (int)rows, (int)K, swiglu ? 1 : 0)) return 0;
+  return fn_->gemm_split_floats((int)M, (int)rows, (int)K, swiglu ? 1 : 0);
+}
+
+// Runs the product through chunk sums in the workspace if that is the faster route and it fits.
+bool Kernels::split(Tensor& out, const Tensor& act, const Tensor& w, bool swiglu, const Tensor* workspace) {
+  if (!workspace) return false;
+  const int64_t M = act.dim(0), K = act.dim(1), rows = w.dim(0);
+  const int64_t need = gemm_workspace_floats(M, rows, K, swiglu);
+  if (need == 0 || workspace->dtype != DType::F32 || workspace->numel() < need) return false;
+  call(fn_->gemm_split(out.data, act.data, w.data, (int)M, (int)rows, (int)K, K, out.dim(1), swiglu ? 1 : 0, workspace->data,
+                       workspace->numel(), stream));
+  return true;
+}
+
+Tensor Kernels::gemm(const Tensor& act, const Tensor& w, const Tensor* workspace) {
   expect(act, "activation", dtype_);
   expect(w, "weight", dtype_);
   if (act.shape.size() != 2 || w.shape.size() != 2 || act.dim(1) != w.dim(1))
     throw EngineError("gemm: activation " + act.describe() + " does not fit weight " + w.describe());
   const int64_t M = act.dim(0), K = act.dim(1), N = w.dim(0);
   Tensor out = empty({M, N});
+  if (split(out, act, w, false, workspace)) return out;
   call(fn_->gemm(out.data, act.data, w.data, (int)M, (int)N, (int)K, K, N, 0, stream));
   return out;
 }
 
-Tensor Kernels::gemm_swiglu(const Tensor& act, const Tensor& w) {
+Tensor Kernels::gemm_swiglu(const Tensor& act, const Tensor& w, const Tensor* workspace) {
   expect(act, "activation", dtype_);
   expect(w, "gate/up weight", dtype_);
   if (act.shape.size() != 2 || w.shape.size() != 2 || act.dim(1) != w.dim(1) || w.dim(0) % 2)
     throw EngineError("gemm_swiglu: activation " + act.describe() + " does not fit a gate/up weight " + w.describe());
   const int64_t M = act.dim(0), K = act.dim(1), I = w.dim(0) / 2;
   // One launch where the sizes allow it, else projection and activation one after the other: the same bits.
-  if (!fn_->gemm_swiglu_supported((int)M, (int)I, (int)K)) return swiglu(gemm(act, w));
+  if (!fn_->gemm_swiglu_supported((int)M, (int)I, (int)K)) return swiglu(gemm(act, w, workspace));
   Tensor out = empty({M, I});
+  if (split(out, act, w, true, workspace)) return out;
   call(fn_->gemm_swiglu(out.data, act.data, w.data, (int)M, (int)I, (int)K, K, I, stream));
   return out;
 }

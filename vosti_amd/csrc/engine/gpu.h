@@ -102,8 +102,13 @@ class Kernels {
   Tensor gather_rows(const Tensor& x, const Tensor& rows);
   Tensor to_f32(const Tensor& x);
   void rope_tables(Tensor& cos, Tensor& sin, const Tensor& inv_freq);
-  Tensor gemm(const Tensor& act, const Tensor& w);                 // act @ w^T, w [out, in]
-  Tensor gemm_swiglu(const Tensor& act, const Tensor& w_gate_up);
+  // act @ w^T, w [out, in].  workspace: float32 scratch; with enough of it (gemm_workspace_floats) some sizes
+  // take a faster route to the same bits.
+  Tensor gemm(const Tensor& act, const Tensor& w, const Tensor* workspace = nullptr);
+  Tensor gemm_swiglu(const Tensor& act, const Tensor& w_gate_up, const Tensor* workspace = nullptr);
+  // float32 elements of workspace with which gemm / gemm_swiglu take the route through chunk sums for these
+  // sizes, or 0 where that route does not exist or is the slower one.
+  int64_t gemm_workspace_floats(int64_t M, int64_t rows, int64_t K, bool swiglu = false) const;
   // Head norm, rotation and cache store of [T, (nq + 2 nkv) d] rows; returns q [T, nq, d] (nq > 0).
   Tensor qkv_post(const Tensor& qkv, int nq, int nkv, int d, const Tensor* k_cache, const Tensor* v_cache, int page_size,
                   const Tensor* q_w, const Tensor* k_w, float eps, const Tensor* cos, const Tensor* sin,
@@ -122,6 +127,7 @@ class Kernels {
   void call(int rc) const;
   void expect(const Tensor& t, const char* what, DType dtype, std::vector<int64_t> shape = {}) const;
   int norm_weight(const Tensor& w, const char* what, int64_t n) const;   // 1 if the weight is float32
+  bool split(Tensor& out, const Tensor& act, const Tensor& w, bool swiglu, const Tensor* workspace);
 
   std::string name_;
   DType dtype_;

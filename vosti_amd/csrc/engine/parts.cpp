@@ -239,10 +239,18 @@ class Attention : public Mixer {
     out.emplace_back("attention.prefill_items", m.prefill);
     out.emplace_back("attention.decode_items", m.decode);
   }
+  // Workspace with which the two projections of T rows take their faster route, where there is one.
+  int64_t gemm_floats(int64_t T) const {
+    return std::max(kernels.gemm_workspace_floats(T, (int64_t)(nq_ + 2 * nkv_) * d_, hidden_),
+                    kernels.gemm_workspace_floats(T, hidden_, (int64_t)nq_ * d_));
+  }
   int64_t workspace_floats(HostStep& step) override {
     AttentionItems& m = items(step);
-    if (m.decode.shape[0] == 0) return 0;
-    return kernels.attn_scratch_floats((int)m.decode.shape[0], nq_, d_, m.nseg);
+    int64_t T = 0;
+    for (int q : step.q_lens) T += q;
+    int64_t need = gemm_floats(T);
+    if (m.decode.shape[0]) need = std::max(need, kernels.attn_scratch_floats((int)m.decode.shape[0], nq_, d_, m.nseg));
+    return need;
   }
 
   Tensor forward(const Tensor& x, StepContext& ctx, CacheEntry& cache) override {
@@ -251,7 +259,13 @@ class Attention : public Mixer {
     const int64_t T = x.dim(0);
     GroupTables& tables = ctx.groups.at(cache.group);
     // Without a cache of its own the keys and values are an earlier execution's: only q is projected.
-    const Tensor qkv = k.gemm(x, cache.writable ? w_qkv_ : w_qkv_.rows(0, (int64_t)nq_ * d_));
+    // The projections, the attention of decoded tokens and the next projection use the step's workspace one
+    // after the other.
+    const int64_t gf = gemm_floats(T);
+    Tensor ws_t;
+    if (gf) ws_t = ctx.workspace(gf);
+    const Tensor* ws = gf ? &ws_t : nullptr;
+    const Tensor qkv = k.gemm(x, cache.writable ? w_qkv_ : w_qkv_.rows(0, (int64_t)nq_ * d_), ws);
     const Norm* en = q_norm_ ? q_norm_.get() : k_norm_.get();
     Tensor q = k.qkv_post(qkv, nq_, cache.writable ? nkv_ : 0, d_, &cache.k, &cache.v, cache.page_size,
                           q_norm_ ? q_norm_->row_scale_weight() : nullptr, k_norm_ ? k_norm_->row_scale_weight() : nullptr,
@@ -269,7 +283,7 @@ class Attention : public Mixer {
       k.paged_attention(out, q, cache.k, cache.v, tables.block_table, ctx.cu_q, ctx.k_len, decode_items, 1, scale_, window_,
                         m.decode_bound, m.nseg, &scratch);
     }
-    return k.gemm(out.view({T, (int64_t)nq_ * d_}), w_o_);
+    return k.gemm(out.view({T, (int64_t)nq_ * d_}), w_o_, ws);
   }
 
  private:
@@ -295,7 +309,20 @@ class SwiGLU : public FeedForward {
     w_gate_up_ = stack_rows({need(t, "gate_proj.weight"), need(t, "up_proj.weight")});
     w_down_ = need(t, "down_proj.weight");
   }
-  Tensor forward(const Tensor& x, StepContext&) override { return kernels.gemm(kernels.gemm_swiglu(x, w_gate_up_), w_down_); }
+  int64_t gemm_floats(int64_t T) const {
+    return std::max(kernels.gemm_workspace_floats(T, 2 * inter_, hidden_, true), kernels.gemm_workspace_floats(T, hidden_, inter_));
+  }
+  int64_t workspace_floats(HostStep& step) override {
+    int64_t T = 0;
+    for (int q : step.q_lens) T += q;
+    return gemm_floats(T);
+  }
+  Tensor forward(const Tensor& x, StepContext& ctx) override {
+    const int64_t n = gemm_floats(x.dim(0));
+    Tensor ws;
+    if (n) ws = ctx.workspace(n);
+    return kernels.gemm(kernels.gemm_swiglu(x, w_gate_up_, n ? &ws : nullptr), w_down_, n ? &ws : nullptr);
+  }
 
  private:
   int64_t hidden_, inter_;

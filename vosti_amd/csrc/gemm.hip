@@ -912,6 +912,131 @@ static int launch_mid(elem_t* out, const elem_t* act, const elem_t* w, int M, in
   return vk_check_launch("gemm_mid");
 }
 
+static int device_cus();
+
+// ---------------------------------------------------------------- split
+// 17 to 64 rows and few weight rows: the kernels above give such a product a workgroup or less per compute
+// unit, each walking a long stretch of K on its own with a window of loads that one latency drains.  Here
+// a workgroup takes 16 NTW weight rows of ONE chunk: a wave's 16 rows x 512 elements are all in flight at
+// once, the chunk of the activations goes into LDS once for its waves, and the chunk sums go to a
+// workspace [chunk][weight tile][activation tile][lane]; a second kernel adds them in chunk order to a
+// zero total, which is what every other kernel computes, and writes the output (with SWIGLU: of
+// silu(g) * u, g and u rounded to the element type first).  16-bit elements only.
+#ifdef VK_BF16
+template <int MT, int NTW>
+__global__ __launch_bounds__(64 * NTW) void gemm_split_kernel(f32x4* __restrict__ partial, const elem_t* __restrict__ act,
+                                                              const elem_t* __restrict__ w, int M, int N, int K,
+                                                              int64_t lda, int ntiles16) {
+  constexpr int ROW_B = KC * (int)sizeof(elem_t);           // bytes of an activation row of a chunk: 1024
+  static_assert(ROW_B == 64 * 16, "a wave-level load fills one activation row");
+  __shared__ __attribute__((aligned(16))) unsigned char lds[16 * MT * ROW_B];
+
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r16 = lane & 15, kg = lane >> 4;
+  const int c = blockIdx.y;
+  const int tile = blockIdx.x * NTW + wave;                  // 16-row weight tile; beyond the last: clamped rows, nothing stored
+
+  // Activations first: row r of the chunk lies at lds + r * 1024, its logical 16-byte column j at physical
+  // column j ^ (r % 16); lane i of a wave-level load fills physical column i.
+#pragma unroll
+  for (int j = 0; j < 16 * MT / NTW; ++j) {
+    const int r = wave + j * NTW;
+    __builtin_amdgcn_global_load_lds(act + (int64_t)min(r, M - 1) * lda + (int64_t)c * KC + ((lane ^ (r & 15)) * VK_VEC),
+                                     (__attribute__((address_space(3))) void*)(lds + r * ROW_B), 16, 0, 0);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  const elem_t* wrow = w + (int64_t)min(tile * 16 + r16, N - 1) * K + (int64_t)c * KC + kg * VK_VEC;
+  frag_t wbuf[KC_SLABS];
+#pragma unroll
+  for (int s = 0; s < KC_SLABS; ++s) wbuf[s] = *reinterpret_cast<const frag_t*>(wrow + s * VK_SLAB);
+  __builtin_amdgcn_sched_barrier(0);
+  static_assert(KC_SLABS == 16, "vmcnt(16) below: the weight loads are the 16 issued last");
+  __builtin_amdgcn_s_waitcnt(0x4F70);      // vmcnt(16): this wave's activation rows are in LDS; its weights still fly
+  __syncthreads();
+
+  f32x4 acc[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int s = 0; s < KC_SLABS; ++s) {
+    frag_t fa[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+      fa[mt] = *reinterpret_cast<const frag_t*>(lds + (mt * 16 + r16) * ROW_B + (((s * 4 + kg) ^ r16) << 4));
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[mt] = mma_slab(wbuf[s], fa[mt], acc[mt]);
+  }
+  if (tile < ntiles16) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) partial[(((int64_t)c * ntiles16 + tile) * MT + mt) * 64 + lane] = acc[mt];
+  }
+}
+
+// One thread per (weight tile, activation tile, lane): the chunk sums in chunk order.  up_tiles > 0: the
+// tile and the one up_tiles after it are the gate and the up projection of the same output columns.
+template <int MT>
+__global__ __launch_bounds__(256) void gemm_split_reduce_kernel(elem_t* __restrict__ out, const f32x4* __restrict__ partial,
+                                                                int M, int N, int64_t ldo, int nchunks, int ntiles16,
+                                                                int up_tiles, int out_vec_ok) {
+  const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int lane = (int)(t & 63), mt = (int)((t >> 6) % MT);
+  const int tile = (int)(t / (64 * MT));
+  const int out_tiles = up_tiles > 0 ? up_tiles : ntiles16;
+  if (tile >= out_tiles) return;
+  const int r16 = lane & 15, kg = lane >> 4;
+  auto sum = [&](int tl) {
+    f32x4 total = {0.f, 0.f, 0.f, 0.f};
+    const f32x4* p0 = partial + ((int64_t)tl * MT + mt) * 64 + lane;
+    const int64_t stride = (int64_t)ntiles16 * MT * 64;
+    int c = 0;
+    for (; c + 8 <= nchunks; c += 8) {         // eight loads in flight, added in chunk order
+      f32x4 p[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) p[i] = p0[(c + i) * stride];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        total.x = total.x + p[i].x; total.y = total.y + p[i].y; total.z = total.z + p[i].z; total.w = total.w + p[i].w;
+      }
+    }
+    for (; c < nchunks; ++c) {
+      const f32x4 p = p0[c * stride];
+      total.x = total.x + p.x; total.y = total.y + p.y; total.z = total.z + p.z; total.w = total.w + p.w;
+    }
+    return total;
+  };
+  f32x4 y = sum(tile);
+  if (up_tiles > 0) {
+    const f32x4 o = sum(tile + up_tiles);
+    const float g[4] = {round_to_elem(y.x), round_to_elem(y.y), round_to_elem(y.z), round_to_elem(y.w)};
+    const float u[4] = {round_to_elem(o.x), round_to_elem(o.y), round_to_elem(o.z), round_to_elem(o.w)};
+    y.x = (g[0] * (1.0f / (1.0f + expf(-g[0])))) * u[0];
+    y.y = (g[1] * (1.0f / (1.0f + expf(-g[1])))) * u[1];
+    y.z = (g[2] * (1.0f / (1.0f + expf(-g[2])))) * u[2];
+    y.w = (g[3] * (1.0f / (1.0f + expf(-g[3])))) * u[3];
+  }
+  store_out4(out, ldo, mt * 16 + r16, tile * 16 + 4 * kg, M, N, y, out_vec_ok);
+}
+
+template <int MT>
+static int launch_split(elem_t* out, const elem_t* act, const elem_t* w, int M, int rows, int K, int64_t lda, int64_t ldo,
+                        int swiglu, float* workspace, int vec_ok, hipStream_t st) {
+  const int ntiles16 = (rows + 15) / 16, nchunks = K / KC;
+  f32x4* partial = reinterpret_cast<f32x4*>(workspace);
+  // Eight waves a workgroup where that still leaves two workgroups or more per compute unit, else four
+  // (64 rows, 4096 x 12288: 37.3 against 35.7 us; 6144 x 4096: 19.1 against 19.9 us; sixteen waves were slower).
+  if ((int64_t)((ntiles16 + 7) / 8) * nchunks >= 2 * device_cus())
+    gemm_split_kernel<MT, 8><<<dim3((ntiles16 + 7) / 8, nchunks), 512, 0, st>>>(partial, act, w, M, rows, K, lda, ntiles16);
+  else
+    gemm_split_kernel<MT, 4><<<dim3((ntiles16 + 3) / 4, nchunks), 256, 0, st>>>(partial, act, w, M, rows, K, lda, ntiles16);
+  const int up_tiles = swiglu ? ntiles16 / 2 : 0;
+  const int out_tiles = swiglu ? up_tiles : ntiles16;
+  const int64_t threads = (int64_t)out_tiles * MT * 64;
+  gemm_split_reduce_kernel<MT><<<(unsigned)((threads + 255) / 256), 256, 0, st>>>(out, partial, M, swiglu ? rows / 2 : rows, ldo,
+                                                                                  nchunks, ntiles16, up_tiles, vec_ok);
+  return vk_check_launch("gemm_split");
+}
+#endif
+
 // ==================================================================== host
 static int device_cus() {
   static int cus = 0;
@@ -1129,6 +1254,56 @@ int vk_gemm_swiglu(elem_t* out, const elem_t* act, const elem_t* w, int M, int I
     SWIGLU_STREAM(8, 1, 1);
 #undef SWIGLU_STREAM
   return vk_check_launch("gemm_swiglu");
+}
+
+
+// float32 elements of workspace that vk_gemm_split needs for these sizes, or 0 if it does not take them:
+// 17 to 64 rows of 16-bit elements, K in whole chunks; rows: weight rows (with swiglu: gate and up rows
+// together, an even number of 16-row tiles).
+int64_t vk_gemm_split_floats(int M, int rows, int K, int swiglu) {
+#ifdef VK_BF16
+  if (M <= 16 || M > 64 || rows <= 0 || K <= 0 || K % KC != 0) return 0;
+  if (swiglu && rows % 32 != 0) return 0;
+  const int mt = (M + 15) / 16;
+  return (int64_t)(K / KC) * ((rows + 15) / 16) * mt * 256;
+#else
+  (void)M; (void)rows; (void)K; (void)swiglu;
+  return 0;
+#endif
+}
+
+// 1 if the route through chunk sums is the faster one for these sizes (measured on Qwen3-8B shapes, MI355X,
+// 64 rows: 4096 x 12288 45 -> 32 us, 6144 x 4096 20.6 -> 18.2 us, 4096 x 4096 16.0 -> 13.8 us; 32 rows:
+// 41 -> 27, 17.8 -> 14.7, 13.4 -> 11.7 us).  Not with the activation folded in (24576 x 4096: 60 -> 62 us), not
+// for small matrices (1000 x 1024 at 32 rows: 4.8 -> 6.5 us), and not for very many weight rows, where the
+// other kernels have workgroups enough and the chunk sums would be a large share of the traffic.
+int vk_gemm_split_preferred(int M, int rows, int K, int swiglu) {
+  if (swiglu || vk_gemm_split_floats(M, rows, K, swiglu) == 0) return 0;
+  return (int64_t)rows * K >= ((int64_t)1 << 23) && rows <= 8192;
+}
+
+// out = act w^T (swiglu 0: w [rows, K], out [M, rows]) or silu(act w_gate^T) * (act w_up^T) (swiglu 1:
+// w = [gate rows; up rows], out [M, rows / 2]), through chunk sums in a workspace: the bits of vk_gemm and
+// vk_gemm_swiglu.  Calls that overlap in time need workspaces of their own.
+int vk_gemm_split(elem_t* out, const elem_t* act, const elem_t* w, int M, int rows, int K, int64_t lda, int64_t ldo,
+                  int swiglu, float* workspace, int64_t workspace_floats, hipStream_t st) {
+  const int64_t need = vk_gemm_split_floats(M, rows, K, swiglu);
+  VK_REQUIRE(need > 0, "gemm_split: sizes M=%d rows=%d K=%d are not supported", M, rows, K);
+  VK_REQUIRE(workspace != nullptr && workspace_floats >= need && ((uintptr_t)workspace % 16) == 0,
+             "gemm_split: a 16-byte aligned workspace of %lld floats is needed", (long long)need);
+  const int out_cols = swiglu ? rows / 2 : rows;
+  VK_REQUIRE(lda >= K && lda % VK_VEC == 0 && ldo >= out_cols, "gemm_split: bad row strides");
+  VK_REQUIRE(((uintptr_t)act % 16) == 0 && ((uintptr_t)w % 16) == 0, "gemm_split: operands must be 16-byte aligned");
+#ifdef VK_BF16
+  const int vec_ok = (ldo % 4 == 0) && ((uintptr_t)out % 16 == 0);
+  const int mt = (M + 15) / 16;
+  if (mt == 2) return launch_split<2>(out, act, w, M, rows, K, lda, ldo, swiglu, workspace, vec_ok, st);
+  if (mt == 3) return launch_split<3>(out, act, w, M, rows, K, lda, ldo, swiglu, workspace, vec_ok, st);
+  return launch_split<4>(out, act, w, M, rows, K, lda, ldo, swiglu, workspace, vec_ok, st);
+#else
+  (void)out; (void)st;
+  return vk_fail("gemm_split: built for 16-bit elements only");
+#endif
 }
 
 }  // extern "C"

@@ -15,7 +15,7 @@ import torch
 
 from . import build
 
-ABI_VERSION = 11
+ABI_VERSION = 12
 SEGMENT_KEYS = 256
 ATTN_ITEM_ROWS = 128      # rows of one prompt item of paged_attention
 
@@ -68,6 +68,10 @@ class Kernels:
         _sig(lib.vk_gemm, P, P, P, I, I, I, L, L, I, P)
         _sig(lib.vk_gemm_swiglu, P, P, P, I, I, I, L, L, P)
         _sig(lib.vk_gemm_swiglu_supported, I, I, I)
+        _sig(lib.vk_gemm_split, P, P, P, I, I, I, L, L, I, P, L, P)
+        lib.vk_gemm_split_floats.argtypes = [I, I, I, I]
+        lib.vk_gemm_split_floats.restype = c_int64
+        _sig(lib.vk_gemm_split_preferred, I, I, I, I)
         _sig(lib.vk_qkv_post, P, L, P, P, P, P, P, I, P, P, I, P, P, I, I, I, I, I, F, P)
         _sig(lib.vk_paged_attention, P, P, P, P, P, I, P, P, P, I, I, I, P, I, I, I, I, I, I, F, P)
         _sig(lib.vk_sample, P, P, P, P, P, I, I, L, P)
@@ -196,10 +200,37 @@ class Kernels:
         self._call(self.lib.vk_fill_random, self._elem(out, "out"), out.numel(), c_uint64(seed & (2**64 - 1)), kind,
                    float(p0), float(p1), self._stream())
 
-    def gemm(self, act: torch.Tensor, w: torch.Tensor, out: torch.Tensor | None = None, kernel: int = 0) -> torch.Tensor:
+    def gemm_workspace_floats(self, M: int, rows: int, K: int, swiglu: bool = False, force: bool = False) -> int:
+        """float32 elements of workspace with which ``gemm`` / ``gemm_swiglu`` take the route through chunk
+        sums for these sizes, or 0 where that route does not exist or is the slower one (``force``: where it
+        does not exist).  A part adds this to what it asks of the step's workspace."""
+        if not force and not self.lib.vk_gemm_split_preferred(M, rows, K, 1 if swiglu else 0):
+            return 0
+        return int(self.lib.vk_gemm_split_floats(M, rows, K, 1 if swiglu else 0))
+
+    def _split(self, out, act, w, M, rows, K, lda, ldo, swiglu, workspace, force=False) -> bool:
+        """Runs the product through chunk sums in ``workspace`` if that is the faster route and it fits."""
+        if workspace is None:
+            if force:
+                raise KernelError("gemm: the route through chunk sums needs a workspace")
+            return False
+        need = self.gemm_workspace_floats(M, rows, K, swiglu, force)
+        if need == 0 or workspace.numel() < need:
+            if force:
+                raise KernelError(f"gemm: no route through chunk sums for M={M} rows={rows} K={K}, or the workspace "
+                                  f"of {workspace.numel()} floats is smaller than {need}")
+            return False
+        self._call(self.lib.vk_gemm_split, out.data_ptr(), act.data_ptr(), w.data_ptr(), M, rows, K, lda, ldo,
+                   1 if swiglu else 0, self._f32(workspace, "workspace"), workspace.numel(), self._stream())
+        return True
+
+    def gemm(self, act: torch.Tensor, w: torch.Tensor, out: torch.Tensor | None = None, kernel: int = 0,
+             workspace: torch.Tensor | None = None) -> torch.Tensor:
         """out = act @ w.T with w in [out_features, in_features] layout.
 
-        ``act`` may be a view of rows with a row stride (its last axis contiguous)."""
+        ``act`` may be a view of rows with a row stride (its last axis contiguous).  ``workspace``: float32
+        scratch; with enough of it (``gemm_workspace_floats``) some sizes take a faster route to the same
+        bits.  ``kernel`` 14 forces that route (tests)."""
         M, K = act.shape
         N, K2 = w.shape
         if K2 != K:
@@ -210,25 +241,31 @@ class Kernels:
         lda = act.stride(0) if M > 1 else max(K, act.stride(0))
         out = self.empty(M, N) if out is None else out
         self._elem(out, "out", M, N)
+        if kernel in (0, 14) and self._split(out, act, w, M, N, K, lda, N, False, workspace, force=kernel == 14):
+            return out
         self._call(self.lib.vk_gemm, out.data_ptr(), act.data_ptr(), w.data_ptr(), M, N, K, lda, N, kernel,
                    self._stream())
         return out
 
-    def gemm_swiglu(self, act: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
+    def gemm_swiglu(self, act: torch.Tensor, w_gate_up: torch.Tensor, workspace: torch.Tensor | None = None,
+                    split: bool = False) -> torch.Tensor:
         """silu(act @ w_gate.T) * (act @ w_up.T) with w_gate_up = [gate rows; up rows].
 
         One launch where the sizes allow it, else the projection and the activation one after the
-        other; the result is the same bits either way."""
+        other; the result is the same bits either way.  ``split`` forces the route through chunk sums in
+        ``workspace`` (tests)."""
         M, K = act.shape
         N2, K2 = w_gate_up.shape
         if K2 != K or N2 % 2:
             raise KernelError(f"gemm_swiglu: activation [{M}, {K}] does not fit a gate/up weight [{N2}, {K2}]")
         I = N2 // 2
         if not (act.is_contiguous() and self.lib.vk_gemm_swiglu_supported(M, I, K)):
-            return self.swiglu(self.gemm(act, w_gate_up))
+            return self.swiglu(self.gemm(act, w_gate_up, workspace=workspace))
         self._elem(act, "activation", M, K)
         self._elem(w_gate_up, "weight", N2, K)
         out = self.empty(M, I)
+        if self._split(out, act, w_gate_up, M, N2, K, K, I, True, workspace, force=split):
+            return out
         self._call(self.lib.vk_gemm_swiglu, out.data_ptr(), act.data_ptr(), w_gate_up.data_ptr(), M, I, K, K, I,
                    self._stream())
         return out

@@ -190,22 +190,33 @@ class Attention(Mixer):
     def step_inputs(self, step: HostStep):
         return self._items_arrays(step)
 
+    def _gemm_floats(self, T: int) -> int:
+        """Workspace with which the two projections of T rows take their faster route, where there is one."""
+        k, H = self.kernels, self.hidden_size
+        return max(k.gemm_workspace_floats(T, (self.nq + 2 * self.nkv) * self.d, H),
+                   k.gemm_workspace_floats(T, H, self.nq * self.d))
+
     def workspace_floats(self, step: HostStep) -> int:
         m = self._items(step)
-        if not m["decode"].shape[0]:
-            return 0
-        return self.kernels.attn_scratch_floats(m["decode"].shape[0], self.nq, self.d, m["nseg"])
+        need = self._gemm_floats(sum(step.q_lens))
+        if m["decode"].shape[0]:
+            need = max(need, self.kernels.attn_scratch_floats(m["decode"].shape[0], self.nq, self.d, m["nseg"]))
+        return need
 
     def forward(self, x: torch.Tensor, ctx: StepContext, cache: PagedKV) -> torch.Tensor:
         k = self.kernels
         T = x.shape[0]
         nq, nkv, d = self.nq, self.nkv, self.d
         tables = ctx.groups[cache.group]
+        # The projections, the attention of decoded tokens and the next projection use the step's workspace
+        # one after the other.
+        gemm_floats = self._gemm_floats(T)
+        ws = ctx.workspace(gemm_floats) if gemm_floats and ctx.workspace is not None else None
         if cache.writable:
-            qkv = k.gemm(x, self.w_qkv)
+            qkv = k.gemm(x, self.w_qkv, workspace=ws)
         else:
             # The keys and values are an earlier execution's: only q is projected.
-            qkv = k.gemm(x, self.w_qkv[: nq * d])
+            qkv = k.gemm(x, self.w_qkv[: nq * d], workspace=ws)
         if self._fused:
             pos = self.position
             q = k.qkv_post(qkv, nq=nq, nkv=nkv if cache.writable else 0, d=d, q_out=None,
@@ -229,7 +240,7 @@ class Attention(Mixer):
             k.paged_attention(q, cache.k, cache.v, tables.block_table, ctx.cu_q, ctx.k_len, decode_items, mode=1,
                               scale=self.scale, window=self.window, max_k_len=m["decode_bound"], nseg=nseg,
                               scratch=scratch, out=out)
-        return k.gemm(out.view(T, nq * d), self.w_o)
+        return k.gemm(out.view(T, nq * d), self.w_o, workspace=ws)
 
     def _unfused(self, qkv, ctx, cache, tables):
         """Norm, position encoding and store as separate steps, for parts that are not RMSNorm / Rotary."""
@@ -279,9 +290,19 @@ class SwiGLU(FeedForward):
         self.w_gate_up = torch.cat([tensors["gate_proj.weight"], tensors["up_proj.weight"]], dim=0).contiguous()
         self.w_down = tensors["down_proj.weight"]
 
+    def _gemm_floats(self, T: int) -> int:
+        k = self.kernels
+        return max(k.gemm_workspace_floats(T, 2 * self.intermediate_size, self.hidden_size, swiglu=True),
+                   k.gemm_workspace_floats(T, self.hidden_size, self.intermediate_size))
+
+    def workspace_floats(self, step: HostStep) -> int:
+        return self._gemm_floats(sum(step.q_lens))
+
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         k = self.kernels
-        return k.gemm(k.gemm_swiglu(x, self.w_gate_up), self.w_down)
+        n = self._gemm_floats(x.shape[0])
+        ws = ctx.workspace(n) if n and ctx is not None and ctx.workspace is not None else None
+        return k.gemm(k.gemm_swiglu(x, self.w_gate_up, workspace=ws), self.w_down, workspace=ws)
 
 
 @register_part("block", "prenorm")
