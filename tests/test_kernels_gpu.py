@@ -553,12 +553,14 @@ def test_attention_refuses_bad_sizes():
 @pytest.mark.parametrize("M,I,K", [(8, 100, 1024), (16, 256, 4096), (1, 33, 512), (5, 48, 96), (20, 64, 1024),
                                    (100, 100, 1024), (300, 256, 2048), (129, 70, 192), (130, 64, 96), (40, 8200, 128),
                                    (8, 100, 5120), (16, 48, 8192), (3, 64, 4608), (32, 4100, 4096), (17, 33, 512),
-                                   (64, 200, 1024), (33, 64, 5120), (48, 8200, 512), (20, 130, 4608), (200, 4200, 128), (515, 4500, 64)])
+                                   (64, 200, 1024), (33, 64, 5120), (48, 8200, 512), (20, 130, 4608), (200, 4200, 128), (515, 4500, 64),
+                                   (40, 16384, 512)])
 def test_gemm_swiglu_fused_equals_separate(dtype, M, I, K):
     """The gate/up projection with the activation folded in (the streaming kernel for few rows, the
     pipelined tile kernel for many, the kernel that shares activations through LDS between them) gives
     the bits of the two separate kernels; (5, 48, 96), (20, 64, 1024)... with K no multiple of 512 and
-    (130, 64, 96) fall back to them."""
+    (130, 64, 96) fall back to them.  Between 17 and 64 rows a workgroup takes two, three or four gate
+    tiles, whichever fills the compute units best: (64, 200, 1024), (48, 8200, 512) and (40, 16384, 512)."""
     k = kern(dtype)
     a, w = rand((M, K), dtype, 1).cuda(), rand((2 * I, K), dtype, 2, K ** -0.5).cuda()    # projections of order 1
     got = k.gemm_swiglu(a, w)

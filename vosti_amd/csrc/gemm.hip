@@ -734,15 +734,19 @@ __device__ __forceinline__ void mid_load_to_lds16(const elem_t* src, unsigned ch
   __builtin_amdgcn_global_load_lds(src, (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
 }
 
-// SWIGLU (one chunk in work, KH = 1): w holds N gate rows, then N up rows; waves 0..3 take four gate
-// tiles, waves 4..7 the matching up tiles, and out[m, n] = silu(g) * u with g and u rounded to the
-// element type first, as the separate kernels compute it.
-template <int MT, int KH, bool SWIGLU = false>
+// SWIGLU (one chunk in work, KH = 1): w holds N gate rows, then N up rows; waves 0..GT-1 take GT gate
+// tiles, waves GT..2GT-1 the matching up tiles, and out[m, n] = silu(g) * u with g and u rounded to the
+// element type first, as the separate kernels compute it.  With GT < 4 the other waves only help to bring
+// in the activations: 12288 gate rows are 256 workgroups of three tiles, one for every compute unit,
+// where four tiles a workgroup leave a quarter of them idle.
+template <int MT, int KH, bool SWIGLU = false, int GT = 4>
 __global__ __launch_bounds__(512) void gemm_mid_kernel(elem_t* __restrict__ out, const elem_t* __restrict__ act,
                                                        const elem_t* __restrict__ w, int M, int N, int K,
                                                        int64_t lda, int64_t ldo, int out_vec_ok) {
   static_assert(!SWIGLU || KH == 1, "the SwiGLU epilogue pairs the waves of one chunk");
-  constexpr int NTW = 8 / KH;                       // weight tiles of the workgroup (16 rows each)
+  static_assert(GT == 4 || (SWIGLU && GT >= 2 && GT < 4), "fewer gate tiles only with the SwiGLU epilogue");
+  constexpr int NTW = 8 / KH;                       // waves side by side along the weight rows
+  constexpr int ACTIVE = SWIGLU ? 2 * GT : 8;       // waves that stream weights
   constexpr int STEPS = KC_SLABS / MID_QS;          // steps per chunk
   constexpr int ROW_B = MID_QS * 64;                // bytes of an activation row in a step: 256
   constexpr int HALF_B = 16 * MT * ROW_B;           // one chunk's part of a buffer
@@ -755,6 +759,7 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(elem_t* __restrict__ out,
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r16 = lane & 15, kg = lane >> 4;
   const int nt = wave % NTW, kh = wave / NTW;
+  const bool active = ACTIVE == 8 || wave < ACTIVE;
   const int row0 = blockIdx.y * 16 * MT;            // more than 16 MT rows: one block of them per blockIdx.y
   const int nchunks = K / KC, ngroups = (nchunks + KH - 1) / KH;     // group: KH chunks in work together
   const int nsteps = ngroups * STEPS;
@@ -762,8 +767,8 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(elem_t* __restrict__ out,
 
   // Weights: row of this wave's tile, chunk sequence kh, kh + KH, ...; a chunk beyond the last is read as
   // the last (and not used), so that every wave issues the same number of loads.
-  const int out_col0 = SWIGLU ? (int)blockIdx.x * 64 + (nt & 3) * 16 : (int)blockIdx.x * 16 * NTW + nt * 16;
-  const int64_t wrow_i = SWIGLU ? (int64_t)(nt >> 2) * N + min(out_col0 + r16, N - 1) : min(out_col0 + r16, N - 1);
+  const int out_col0 = SWIGLU ? (int)blockIdx.x * 16 * GT + (nt % GT) * 16 : (int)blockIdx.x * 16 * NTW + nt * 16;
+  const int64_t wrow_i = SWIGLU ? (int64_t)min(nt / GT, 1) * N + min(out_col0 + r16, N - 1) : min(out_col0 + r16, N - 1);
   const elem_t* wrow = w + wrow_i * K + kg * VK_VEC;
   frag_t wbuf[MID_W];
   auto issue_w = [&](int g, int slot) {              // g: this wave's slab number; slot = g % MID_W
@@ -814,48 +819,58 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(elem_t* __restrict__ out,
     }
   };
 
-  issue_a(0);
-  __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-  for (int i = 0; i < MID_W; ++i) issue_w(i, i);
-  __builtin_amdgcn_sched_barrier(0);
   constexpr int TURN = MID_W / MID_QS;      // steps in one turn of the weight window
   static_assert(STEPS % TURN == 0, "a turn of the weight window is a whole number of steps");
-  for (int t2 = 0; t2 < nsteps; t2 += TURN) {
+  issue_a(0);
+  __builtin_amdgcn_sched_barrier(0);
+  if (active) {
 #pragma unroll
-   for (int u = 0; u < TURN; ++u) {         // written out: the window's slots are then fixed registers
-    const int t = t2 + u;
-    if (t == 0) mid_wait_vmcnt_w(); else mid_wait_vmcnt_4();
-    mid_barrier();          // step t's activations are in LDS; everyone is done with the other buffer
-    const int group = t / STEPS, q = t % STEPS;
-    if (q == 0 && group > 0) {
-      if (kh == 0) close_group(KH);           // the group before is complete
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-    }
+    for (int i = 0; i < MID_W; ++i) issue_w(i, i);
     __builtin_amdgcn_sched_barrier(0);
-    issue_a(t + 1);
-    __builtin_amdgcn_sched_barrier(0);
-    const unsigned char* abase = lds + (t & 1) * BUF_B + kh * HALF_B;
+    for (int t2 = 0; t2 < nsteps; t2 += TURN) {
 #pragma unroll
-    for (int s = 0; s < MID_QS; ++s) {
-      const int g = t * MID_QS + s;
-      const frag_t fw = wbuf[u * MID_QS + s];
-      frag_t fa[MT];
+      for (int u = 0; u < TURN; ++u) {         // written out: the window's slots are then fixed registers
+        const int t = t2 + u;
+        if (t == 0) mid_wait_vmcnt_w(); else mid_wait_vmcnt_4();
+        mid_barrier();          // step t's activations are in LDS; everyone is done with the other buffer
+        const int group = t / STEPS, q = t % STEPS;
+        if (q == 0 && group > 0) {
+          if (kh == 0) close_group(KH);           // the group before is complete
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-        fa[mt] = *reinterpret_cast<const frag_t*>(abase + (mt * 16 + r16) * ROW_B + (((s * 4 + kg) ^ r16) << 4));
-      issue_w(g + MID_W, u * MID_QS + s);
+          for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        issue_a(t + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        const unsigned char* abase = lds + (t & 1) * BUF_B + kh * HALF_B;
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) acc[mt] = mma_slab(fw, fa[mt], acc[mt]);
+        for (int s = 0; s < MID_QS; ++s) {
+          const int g = t * MID_QS + s;
+          const frag_t fw = wbuf[u * MID_QS + s];
+          frag_t fa[MT];
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+            fa[mt] = *reinterpret_cast<const frag_t*>(abase + (mt * 16 + r16) * ROW_B + (((s * 4 + kg) ^ r16) << 4));
+          issue_w(g + MID_W, u * MID_QS + s);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) acc[mt] = mma_slab(fw, fa[mt], acc[mt]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (q == STEPS - 1 && kh > 0) {
+          // This wave's chunk of the group is complete: hand it over (one beyond the last chunk is not used).
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) part[(((kh - 1) * NTW + nt) * MT + mt) * 64 + lane] = acc[mt];
+        }
+      }
     }
-    __builtin_amdgcn_sched_barrier(0);
-    if (q == STEPS - 1 && kh > 0) {
-      // This wave's chunk of the group is complete: hand it over (one beyond the last chunk is not used).
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) part[(((kh - 1) * NTW + nt) * MT + mt) * 64 + lane] = acc[mt];
+  } else {
+    // A wave without weights only brings in its share of the activations: the same barriers, and nothing
+    // in flight but those loads.
+    for (int t = 0; t < nsteps; ++t) {
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+      mid_barrier();
+      issue_a(t + 1);
     }
-   }
   }
   __builtin_amdgcn_s_waitcnt(0x0F70);      // the loads issued beyond the end
   mid_barrier();
@@ -864,13 +879,13 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(elem_t* __restrict__ out,
     if (SWIGLU) {
       // Every wave is past the barrier above, so the activation buffers are free: the up waves leave
       // their sums there for the gate waves of the same columns.
-      f32x4* ex = reinterpret_cast<f32x4*>(lds);       // [4 tiles][MT][64 lanes]
-      if (nt >= 4) {
+      f32x4* ex = reinterpret_cast<f32x4*>(lds);       // [GT tiles][MT][64 lanes]
+      if (nt >= GT && active) {
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) ex[((nt - 4) * MT + mt) * 64 + lane] = total[mt];
+        for (int mt = 0; mt < MT; ++mt) ex[((nt - GT) * MT + mt) * 64 + lane] = total[mt];
       }
       __syncthreads();
-      if (nt < 4) {
+      if (nt < GT) {
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
           const f32x4 t = total[mt], o = ex[(nt * MT + mt) * 64 + lane];
@@ -893,22 +908,22 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(elem_t* __restrict__ out,
 }
 
 // N: weight rows, or with SWIGLU the gate rows (and as many up rows after them).
-template <int MT, int KH, bool SWIGLU = false>
+template <int MT, int KH, bool SWIGLU = false, int GT = 4>
 static int launch_mid(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K, int64_t lda, int64_t ldo,
                       int vec_ok, hipStream_t st) {
   constexpr int NTW = 8 / KH;
-  constexpr int COLS = SWIGLU ? 64 : 16 * NTW;      // output columns of a workgroup
+  constexpr int COLS = SWIGLU ? 16 * GT : 16 * NTW; // output columns of a workgroup
   const size_t smem = (size_t)2 * KH * 16 * MT * (MID_QS * 64) + (size_t)(KH - 1) * NTW * MT * 64 * sizeof(f32x4);
   static_assert(!SWIGLU || 2 * 16 * MT * (MID_QS * 64) >= 4 * MT * 64 * (int)sizeof(f32x4), "the exchange fits the activation buffers");
   static bool configured = false;
   if (!configured) {
-    (void)hipFuncSetAttribute((const void*)gemm_mid_kernel<MT, KH, SWIGLU>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    (void)hipFuncSetAttribute((const void*)gemm_mid_kernel<MT, KH, SWIGLU, GT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     configured = true;
   }
   // Blocks of 16 MT rows side by side: those of a weight tile run at about the same time, and on the same
   // chip part when the grid's width is a multiple of eight, so that all but one find it in its cache.
   const dim3 grid((N + COLS - 1) / COLS, (M + 16 * MT - 1) / (16 * MT));
-  gemm_mid_kernel<MT, KH, SWIGLU><<<grid, 512, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok);
+  gemm_mid_kernel<MT, KH, SWIGLU, GT><<<grid, 512, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok);
   return vk_check_launch("gemm_mid");
 }
 
@@ -1227,7 +1242,25 @@ int vk_gemm_swiglu(elem_t* out, const elem_t* act, const elem_t* w, int M, int I
     return launch_pipe<2, true>(out, act, w, M, I, K, lda, ldo, (ldo % 4 == 0) && ((uintptr_t)out % 16 == 0), st);
   if (how == 3) {
     const int ok4 = (ldo % 4 == 0) && ((uintptr_t)out % 16 == 0);
-    if (M <= 32) return launch_mid<2, 1, true>(out, act, w, M, I, K, lda, ldo, ok4, st);
+    // Gate tiles per workgroup: of four, three and two, the number whose workgroups fill the compute units
+    // best, a workgroup per unit at a time; the larger one where two fill them alike.  64 rows, K = 4096:
+    // 12288 gate rows (192, 256, 384 workgroups) 55.4, 49.7, 58.5 us; 8192 gate rows (128, 171, 256) 52.8, 47.0,
+    // 41.6 us; 17408 gate rows at K = 5120 (272, 363, 544) 127.5, 108.4, 123.2 us.
+    const int tiles = (I + 15) / 16, cus = device_cus();
+    int gt = 4;
+    double best = 0.0;
+    for (int g = 4; g >= 2; --g) {
+      const int wgs = (tiles + g - 1) / g;
+      const double filled = (double)wgs / ((double)((wgs + cus - 1) / cus) * cus);
+      if (filled > best + 1e-9) { best = filled; gt = g; }
+    }
+    if (M <= 32) {
+      if (gt == 3) return launch_mid<2, 1, true, 3>(out, act, w, M, I, K, lda, ldo, ok4, st);
+      if (gt == 2) return launch_mid<2, 1, true, 2>(out, act, w, M, I, K, lda, ldo, ok4, st);
+      return launch_mid<2, 1, true>(out, act, w, M, I, K, lda, ldo, ok4, st);
+    }
+    if (gt == 3) return launch_mid<4, 1, true, 3>(out, act, w, M, I, K, lda, ldo, ok4, st);
+    if (gt == 2) return launch_mid<4, 1, true, 2>(out, act, w, M, I, K, lda, ldo, ok4, st);
     return launch_mid<4, 1, true>(out, act, w, M, I, K, lda, ldo, ok4, st);
   }
   const int ntiles = (I + 15) / 16;
