@@ -521,6 +521,18 @@ __device__ __forceinline__ void pipe_load_to_lds16(const elem_t* src, unsigned c
   __builtin_amdgcn_global_load_lds(src, (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
 }
 
+// The same load with its address in two parts: a base held in scalar registers, the same for every lane, and a
+// 32-bit offset per lane.  The compiler's own form of it adds base and offset in vector registers before every
+// load (it moves what does not change along K out of the loop and is left with a vector sum); written out, the
+// advancing base costs two scalar additions per K tile for all loads together.  lds_addr: the wave's 1 KB
+// block in LDS, below 64 KB.
+__device__ __forceinline__ void pipe_load_to_lds16_sv(const unsigned char* sbase, unsigned voff, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(sbase), "s"(lds_addr) : "memory");     // m0 is the compiler's scratch: it sets it anew before every use of its own
+}
+__device__ __forceinline__ unsigned lds_offset_of(const unsigned char* p) {
+  return (unsigned)(unsigned long)((__attribute__((address_space(3))) const void*)p);
+}
+
 // FNW: 16-row weight fragments per wave, 4 (a workgroup takes 128 weight rows) or 2 (64: twice the
 // workgroups, for grids that would leave compute units with one workgroup or none).
 template <int S, bool WHOLE, bool SWIGLU, int FNW = 4>
@@ -532,7 +544,9 @@ __global__ __launch_bounds__(256, 2) void gemm_pipe_kernel(elem_t* __restrict__ 
   constexpr int W_BYTES = BN * T_ROWB, STAGE_BYTES = W_BYTES + 128 * T_ROWB;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];   // [stage][w tile, act tile]
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // The wave number as a scalar: what depends on it alone (LDS addresses, which rows a load brings)
+  // then needs no vector registers.
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r16 = lane & 15, kg = lane >> 4;
   const int wn = wave & 1, wm = wave >> 1;
   // Workgroups start in the order of their linear index.  That order walks bands of band_w column
@@ -554,25 +568,36 @@ __global__ __launch_bounds__(256, 2) void gemm_pipe_kernel(elem_t* __restrict__ 
   // A wave-level load moves 8 rows x 128 bytes; lane i fills LDS slot i of the 1 KB block, which is
   // row i/8, physical 16-byte column i%8, i.e. logical column (i%8) ^ (i/8).
   const int lr = lane >> 3, lc = (lane & 7) ^ lr;
-  const elem_t* gw[FNW];
-  const elem_t* ga[4];
+  // A load's address is a base that is the same for the whole workgroup (the first weight row of the
+  // block, or of its up rows; the first activation row), which advances along K as a scalar, plus a
+  // 32-bit offset per lane that never changes: no vector arithmetic per load.
+  const unsigned char* wbase = reinterpret_cast<const unsigned char*>(w + (int64_t)min(n_blk, N - 1) * K);
+  const unsigned char* ubase = reinterpret_cast<const unsigned char*>(w + (int64_t)(N + min(n_blk, N - 1)) * K);   // SWIGLU: the up rows
+  const unsigned char* abase = reinterpret_cast<const unsigned char*>(act + (int64_t)min(m_blk, M - 1) * lda);
+  unsigned offw[FNW], offa[4];
 #pragma unroll
   for (int j = 0; j < FNW; ++j) {
     const int row = (wave * FNW + j) * 8 + lr;
-    const int wrow = SWIGLU ? (row < 64 ? min(n_blk + row, N - 1) : N + min(n_blk + row - 64, N - 1)) : min(n_blk + row, N - 1);
-    gw[j] = w + (int64_t)wrow * K + lc * VK_VEC;
+    const int local = SWIGLU ? (row < 64 ? row : row - 64) : row;                 // row of the block, gate or up
+    const int clamped = min(n_blk + local, N - 1) - min(n_blk, N - 1);
+    offw[j] = (unsigned)(((int64_t)clamped * K + lc * VK_VEC) * (int64_t)sizeof(elem_t));
   }
 #pragma unroll
-  for (int j = 0; j < 4; ++j) ga[j] = act + (int64_t)min(m_blk + (wave * 4 + j) * 8 + lr, M - 1) * lda + lc * VK_VEC;
+  for (int j = 0; j < 4; ++j) {
+    const int clamped = min(m_blk + (wave * 4 + j) * 8 + lr, M - 1) - min(m_blk, M - 1);
+    offa[j] = (unsigned)(((int64_t)clamped * lda + lc * VK_VEC) * (int64_t)sizeof(elem_t));
+  }
+  const unsigned lds0 = lds_offset_of(lds);
   auto issue = [&](int kt) {                 // FNW + 4 loads per wave
-    unsigned char* base = lds + (kt % S) * STAGE_BYTES;
-    const int k = kt * 2 * VK_SLAB;
+    const unsigned base = lds0 + (kt % S) * STAGE_BYTES;
+    const int64_t kb = (int64_t)kt * 2 * VK_SLAB * (int64_t)sizeof(elem_t);
 #pragma unroll
-    for (int j = 0; j < FNW; ++j)
-      pipe_load_to_lds16(gw[j] + k, base + (wave * FNW + j) * 8 * T_ROWB);
+    for (int j = 0; j < FNW; ++j) {
+      const bool up = SWIGLU && (wave * FNW + j) * 8 >= 64;       // a scalar: all eight rows of a load are of one kind
+      pipe_load_to_lds16_sv((up ? ubase : wbase) + kb, offw[j], base + (wave * FNW + j) * 8 * T_ROWB);
+    }
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-      pipe_load_to_lds16(ga[j] + k, base + W_BYTES + (wave * 4 + j) * 8 * T_ROWB);
+    for (int j = 0; j < 4; ++j) pipe_load_to_lds16_sv(abase + kb, offa[j], base + W_BYTES + (wave * 4 + j) * 8 * T_ROWB);
   };
 
   f32x4 acc[FNW][4], total[FNW][4];
