@@ -15,6 +15,7 @@ against 8 TB/s; ``points`` holds decode throughput at batch 1 and 64.
 from __future__ import annotations
 
 import argparse
+import os
 import json
 import random
 import sys
@@ -69,6 +70,9 @@ def main() -> int:
     ap.add_argument("--prompt-tokens", type=int, default=PROMPT_TOKENS,
                     help="context length of the decode measurement (the prefill figure is always of 2,048 tokens)")
     ap.add_argument("--workload", default="decode8b", choices=["decode8b", "mixed14b", "prefix32b"])
+    ap.add_argument("--engine", default="native", choices=["native", "python"],
+                    help="which engine runs the timed decode steps: the native one (vosti_amd.engine.NativeEngine, the same "
+                         "kernels, cache manager and scheduler without Python between two steps) or the Python one")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -79,7 +83,8 @@ def main() -> int:
 
     import torch
     from vosti_amd.config import Qwen3Config
-    from vosti_amd.engine import Engine
+    import tempfile
+    from vosti_amd.engine import Engine, NativeEngine
     from vosti_amd.models import build_model
     from vosti_amd.sampling import SamplingParams
     from vosti_amd.weights import random_weights_on_gpu
@@ -102,14 +107,24 @@ def main() -> int:
     def prompt(n=None):
         return [rng.randrange(cfg.vocab_size) for _ in range(prompt_tokens if n is None else n)]
 
-    def decode_run(B: int, steps: int, warmup: int, per_kernel_into: dict | None = None):
-        eng = Engine(model, num_pages=B * pages_per_request, page_size=page, max_num_seqs=B, max_num_batched_tokens=4096,
-                     enable_prefix_cache=False, graphs=bool(args.graphs))
+    native_dir = tempfile.TemporaryDirectory()          # what the native engine is given: config.json; the weights are the same random streams
+    with open(os.path.join(native_dir.name, "config.json"), "w") as f:
+        json.dump(cfg.to_dict(), f)
+
+    def decode_run(B: int, steps: int, warmup: int, per_kernel_into: dict | None = None, which: str | None = None):
+        """Seconds per decode step of B requests at the context length, and the mean context over the timed steps."""
+        which = which or args.engine
+        kw = dict(num_pages=B * pages_per_request, page_size=page, max_num_seqs=B, max_num_batched_tokens=4096,
+                  enable_prefix_cache=False, graphs=bool(args.graphs))
+        if which == "native":
+            eng = NativeEngine(native_dir.name, dtype=args.dtype, random_weights_seed=0, **kw)
+        else:
+            eng = Engine(model, **kw)
         sp = SamplingParams(max_tokens=GENERATED_TOKENS, ignore_eos=True)
         for _ in range(B):
             eng.add_request(prompt(), sp)
-        while eng.scheduler.num_waiting() or any(eng.cache.length(r) < prompt_tokens for r in range(eng._next_id - B, eng._next_id)):
-            eng.step()                                   # prefill, two prompts a step
+        while len(eng.step()) < B:                       # prefill, two prompts a step, beside the decoding of those that are through
+            pass
         for _ in range(warmup):
             assert len(eng.step()) == B
         torch.cuda.synchronize()
@@ -121,7 +136,10 @@ def main() -> int:
         ctx = prompt_tokens + warmup + 1 + (steps - 1) / 2.0          # mean keys per request over the timed steps
         if per_kernel_into is not None:
             try:
-                per_kernel_into["decode"] = kernel_times(model, cfg, eng.pool, B, int(ctx), elem, decode=True)
+                from vosti_amd.cache import CachePool
+                pool = eng.pool if which == "python" else CachePool(model, page_size=page, num_pages=B * pages_per_request, num_slots=B + 1)
+                per_kernel_into["decode"] = kernel_times(model, cfg, pool, B, int(ctx), elem, decode=True)
+                del pool
             except Exception as e:      # the step's own figures stand without these
                 per_kernel_into["decode"] = {"error": f"{type(e).__name__}: {e}"}
         del eng
@@ -158,7 +176,7 @@ def main() -> int:
                    "q_heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
                    "vocab_size": cfg.vocab_size, "global_batch": args.batch, "seq_len": prompt_tokens + GENERATED_TOKENS,
                    "prompt_tokens": prompt_tokens, "context_at_timing": round(ctx), "page_size": page,
-                   "parallelism": "single GPU", "graphs": bool(args.graphs)},
+                   "parallelism": "single GPU", "graphs": bool(args.graphs), "engine": args.engine},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
     }
@@ -171,6 +189,10 @@ def main() -> int:
         for B, name in ((1, "decode_b1"), (64, "decode_b64")):
             s, _ = decode_run(B, min(args.steps, 32), min(args.warmup, 4))
             points[name] = round(B / s, 2)
+        # The same steps through the other engine: what the Python host code between two steps costs.
+        other = "python" if args.engine == "native" else "native"
+        s, _ = decode_run(args.batch, args.steps, args.warmup, which=other)
+        points[f"decode_b{args.batch}_{other}_engine"] = round(args.batch / s, 2)
         record["points"] = points
         if not args.no_per_kernel:
             try:
@@ -275,7 +297,8 @@ def other_workload(args) -> int:
     """The two larger shapes with the workloads named for them: one JSON line each, same fields."""
     import torch
     from vosti_amd.config import Qwen3Config
-    from vosti_amd.engine import Engine
+    import tempfile
+    from vosti_amd.engine import Engine, NativeEngine
     from vosti_amd.models import build_model
     from vosti_amd.sampling import SamplingParams
     from vosti_amd.weights import random_weights_on_gpu

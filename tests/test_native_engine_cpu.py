@@ -92,6 +92,17 @@ def test_missing_keys_defaults_and_zero_layers(program, tmp_path):
     assert describe(program, tmp_path).returncode == 1
 
 
+def test_random_streams_have_the_python_package_seeds(program, tiny_dirs):
+    """The seed of a tensor's random stream is a BLAKE2b digest of "<seed>:<name>"; the program computes it
+    with code of its own."""
+    from vosti_amd.weights.random_init import tensor_seed
+    r = subprocess.run([program, "--kind", "describe", "--model-path", str(tiny_dirs["B"]), "--random-weights", "20250101"],
+                       capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    got = json.loads(r.stdout)
+    assert [int(t) for t in got["tensor_seeds"]] == [tensor_seed(20250101, n) for n in got["tensor_names"]]
+
+
 def test_usage_errors(program, tmp_path):
     r = subprocess.run([program, "--family", "qwen3"], capture_output=True, text=True, env={})
     assert r.returncode == 2 and "MODEL_PATH (or --model-path) is required" in r.stderr

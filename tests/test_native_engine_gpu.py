@@ -131,6 +131,58 @@ def test_shared_prefixes_end_tokens_and_stored_types(program, tiny_dirs, tmp_pat
         ps, SamplingParams(max_tokens=10, eos_token_ids=tuple(eos), ignore_eos=True), arrival_steps=[0, 3, 3])
 
 
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_random_weights_are_the_python_package_s(program, tmp_path, dtype_name):
+    """--random-weights SEED draws on the GPU what the random-model kind of the Python launcher writes for
+    that seed: a folder with nothing but config.json generates the tokens of the written folder.  One line
+    per engine step goes to --step-times."""
+    from vosti_amd.config import Qwen3Config
+    from vosti_amd.sampling import SamplingParams
+    from vosti_amd.weights import write_random_model
+    cfg = Qwen3Config(**TINY["B"][0])
+    written = write_random_model(cfg, 77, tmp_path / "written", DTYPES[dtype_name])
+    bare = tmp_path / "bare"
+    bare.mkdir()
+    shutil.copy(written / "config.json", bare / "config.json")
+    p = prompts("B", [50], seed=2)[0]
+    r = run_native(program, dtype_name, args=["--model-path", str(bare), "--random-weights", "77", "--prompt-ids", ",".join(map(str, p)),
+                                              "--max-tokens", "10", "--num-blocks", "16", "--page-size", "8", "--step-times", str(tmp_path / "times.txt")])
+    out = json.loads([l for l in r.stdout.splitlines() if l.startswith("MODEL_OUTPUT_TOKEN_IDS=")][0].split("=", 1)[1])
+    assert [out] == engine(written, dtype_name, num_pages=16, page_size=8, max_num_seqs=1).generate([p], SamplingParams(max_tokens=10))
+    times = [l.split() for l in (tmp_path / "times.txt").read_text().splitlines()]
+    assert [(int(t[0]), int(t[1]), int(t[2])) for t in times] == [(1, 50, 1)] + [(1, 1, 1)] * 9 and all(float(t[3]) > 0 for t in times)
+
+
+@pytest.mark.parametrize("graphs", [False, True])
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_native_engine_from_python(tiny_dirs, dtype_name, graphs):
+    """NativeEngine is the native engine behind Engine's face: the same requests, the same tokens, in one
+    process with the Python engine (one HIP runtime, one kernel library, streams of their own)."""
+    from vosti_amd.engine import NativeEngine, NativeEngineError
+    from vosti_amd.sampling import SamplingParams
+    ps = prompts("A", [4, 9, 2, 17, 5, 11, 3], seed=31)
+    sp = [SamplingParams(max_tokens=12 + 9 * i, temperature=0.5 * (i % 2), seed=i, ignore_eos=True) for i in range(7)]
+    kw = dict(num_pages=64, page_size=16, max_num_seqs=7, graphs=graphs)
+    want = engine(tiny_dirs["A"], dtype_name, **kw).generate(ps, sp, arrival_steps=[0, 0, 1, 1, 2, 5, 9])
+    native = NativeEngine(tiny_dirs["A"], dtype=dtype_name, **kw)
+    assert native.generate(ps, sp, arrival_steps=[0, 0, 1, 1, 2, 5, 9]) == want
+    st = native.stats()
+    assert st["cache_requests"] == 0 and native.cache_check() == "" and not native.has_unfinished()
+    assert (st["graph_stats"]["replayed"] > 0) == graphs
+    # Step by step, and what it refuses.
+    rid = native.add_request(ps[2], SamplingParams(max_tokens=3))        # a greedy one
+    got = []
+    while native.has_unfinished():
+        got += [t for r, t in native.step().items() if r == rid]
+    assert got == want[2][:3]
+    with pytest.raises(ValueError, match="EmptyPrompt"):
+        native.add_request([], SamplingParams(max_tokens=3))
+    with pytest.raises(ValueError, match="prompt token outside"):
+        native.add_request([10 ** 6], SamplingParams(max_tokens=3))
+    with pytest.raises(NativeEngineError, match="config.json is missing"):
+        NativeEngine("/nonexistent", dtype=dtype_name)
+
+
 def test_one_error_for_weights_that_do_not_fit(program, tiny_dirs, tmp_path):
     d = tmp_path / "model"
     shutil.copytree(tiny_dirs["B"], d)

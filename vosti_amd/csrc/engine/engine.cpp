@@ -1,6 +1,7 @@
 #include "engine.h"
 
 #include <algorithm>
+#include <chrono>
 #include <numeric>
 
 namespace vosti {
@@ -29,7 +30,9 @@ Engine::Engine(const EngineOptions& opt) {
   ModelSpec spec = model_spec_from_dir(opt.model_dir);
   kernels_ = std::make_unique<Kernels>(opt.lib_dir, opt.dtype);
   model_ = std::make_unique<DecoderModel>(std::move(spec), *kernels_);
-  {
+  if (opt.random_weights) {
+    model_->random_weights(opt.random_seed);
+  } else {
     Checkpoint ckpt(opt.model_dir);
     model_->load_weights(ckpt);
   }
@@ -78,6 +81,7 @@ RequestId Engine::add_request(const std::vector<int32_t>& prompt, const Sampling
 }
 
 std::vector<std::pair<RequestId, int32_t>> Engine::step() {
+  const auto t0 = std::chrono::steady_clock::now();
   std::vector<PlanRow> rows;
   std::vector<int32_t> tokens;
   const PlanStatus st = scheduler_->plan(rows, tokens);
@@ -102,6 +106,15 @@ std::vector<std::pair<RequestId, int32_t>> Engine::step() {
     throw EngineError("the scheduler refused " + std::to_string(sampled.size()) + " sampled tokens for a plan with " +
                       std::to_string(scheduler_->num_planned_samples()) + " sampled rows");
   ++steps_;
+  if (record_times_) {
+    StepTime t;
+    t.rows = (int)rows.size();
+    t.tokens = (int)tokens.size();
+    t.sampled = (int)sampled.size();
+    if (sampled.empty()) synchronize();          // a step without a readback has not waited for the GPU yet
+    t.ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+    step_times_.push_back(t);
+  }
   for (const Emitted& e : emitted) {
     out.emplace_back(e.id, e.token);
     if (e.finished) params_.erase(e.id);

@@ -43,6 +43,14 @@ struct EngineOptions {
   bool prefix_cache = true;
   int max_model_len = 0;         // 0: the model's positions
   bool graphs = false;           // VOSTI_CUDA_GRAPH (engine_setup.rs:79-81)
+  bool random_weights = false;   // draw the weights from random_seed on the GPU; the folder needs config.json only
+  uint64_t random_seed = 0;
+};
+
+// What one engine step took, for measurements.
+struct StepTime {
+  int rows = 0, tokens = 0, sampled = 0;
+  double ms = 0.0;               // plan, forward, sample, readback and commit, by the host's clock
 };
 
 class Engine {
@@ -66,6 +74,8 @@ class Engine {
   ModelRunner& runner() { return *runner_; }
   DecoderModel& model() { return *model_; }
   const std::vector<RequestId>& last_scheduled() const { return last_scheduled_; }
+  void record_step_times(bool on) { record_times_ = on; }
+  const std::vector<StepTime>& step_times() const { return step_times_; }
 
  private:
   std::vector<int32_t> forward_and_sample(const std::vector<PlanRow>& rows, const std::vector<int32_t>& tokens);
@@ -84,6 +94,8 @@ class Engine {
   RequestId next_id_ = 0;
   int64_t steps_ = 0;
   std::vector<RequestId> last_scheduled_;
+  bool record_times_ = false;
+  std::vector<StepTime> step_times_;
   // The sampler's buffers: temperatures and uniform numbers up, token ids down.
   float* sample_in_ = nullptr;        // pinned [2, rows]
   int32_t* sample_out_ = nullptr;     // pinned [rows]

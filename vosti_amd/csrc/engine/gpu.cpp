@@ -83,6 +83,7 @@ struct Kernels::Fn {
   int (*gather_rows)(P, CP, CP, int, int, hipStream_t);
   int (*cast_to_f32)(P, CP, int64_t, hipStream_t);
   int (*rope_tables)(P, P, CP, int, int, hipStream_t);
+  int (*fill_random)(P, int64_t, uint64_t, int, float, float, hipStream_t);
   int (*gemm)(P, CP, CP, int, int, int, int64_t, int64_t, int, hipStream_t);
   int (*gemm_swiglu)(P, CP, CP, int, int, int, int64_t, int64_t, hipStream_t);
   int (*gemm_swiglu_supported)(int, int, int);
@@ -118,7 +119,7 @@ Kernels::Kernels(const std::string& lib_dir, const std::string& name) : name_(na
     throw EngineError(path + " has ABI " + std::to_string(fn_->abi_version()) + ", expected " + std::to_string(KERNEL_ABI) + "; rebuild it");
   if (fn_->elem_bytes() != dtype_bytes(dtype_)) throw EngineError(path + " was built for another element type");
   VK(embedding, "vk_embedding"); VK(rmsnorm, "vk_rmsnorm"); VK(add_rmsnorm, "vk_add_rmsnorm"); VK(swiglu, "vk_swiglu");
-  VK(gather_rows, "vk_gather_rows"); VK(cast_to_f32, "vk_cast_to_f32"); VK(rope_tables, "vk_rope_tables");
+  VK(gather_rows, "vk_gather_rows"); VK(cast_to_f32, "vk_cast_to_f32"); VK(rope_tables, "vk_rope_tables"); VK(fill_random, "vk_fill_random");
   VK(gemm, "vk_gemm"); VK(gemm_swiglu, "vk_gemm_swiglu"); VK(gemm_swiglu_supported, "vk_gemm_swiglu_supported");
   VK(gemm_split, "vk_gemm_split"); VK(gemm_split_floats, "vk_gemm_split_floats"); VK(gemm_split_preferred, "vk_gemm_split_preferred");
   VK(qkv_post, "vk_qkv_post"); VK(paged_attention, "vk_paged_attention"); VK(sample, "vk_sample");
@@ -248,6 +249,11 @@ bool Kernels::split(Tensor& out, const Tensor& act, const Tensor& w, bool swiglu
   call(fn_->gemm_split(out.data, act.data, w.data, (int)M, (int)rows, (int)K, K, out.dim(1), swiglu ? 1 : 0, workspace->data,
                        workspace->numel(), stream));
   return true;
+}
+
+void Kernels::fill_random(Tensor& out, uint64_t seed, int kind, float p0, float p1) {
+  expect(out, "tensor to fill", dtype_);
+  call(fn_->fill_random(out.data, out.numel(), seed, kind, p0, p1, stream));
 }
 
 Tensor Kernels::gemm(const Tensor& act, const Tensor& w, const Tensor* workspace) {

@@ -102,6 +102,9 @@ class Kernels {
   Tensor gather_rows(const Tensor& x, const Tensor& rows);
   Tensor to_f32(const Tensor& x);
   void rope_tables(Tensor& cos, Tensor& sin, const Tensor& inv_freq);
+  // Counter-based random fill: element i is a function of (seed, i); kind 0: a sum of four 16-bit uniforms
+  // scaled by p0, kind 1: p0 + u * p1.
+  void fill_random(Tensor& out, uint64_t seed, int kind, float p0, float p1);
   // act @ w^T, w [out, in].  workspace: float32 scratch; with enough of it (gemm_workspace_floats) some sizes
   // take a faster route to the same bits.
   Tensor gemm(const Tensor& act, const Tensor& w, const Tensor* workspace = nullptr);

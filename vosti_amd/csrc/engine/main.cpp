@@ -26,7 +26,9 @@
 // Options without a counterpart in the reference: VOSTI_DTYPE / --dtype (bfloat16, float32),
 // VOSTI_TEMPERATURE / --temperature, VOSTI_SEED / --seed, VOSTI_PAGE_SIZE / --page-size,
 // VOSTI_PREFIX_CACHE / --prefix-cache (0, 1), VOSTI_LIB_DIR / --lib-dir (where the kernel libraries lie;
-// default: beside this program).  End tokens come from generation_config.json's eos_token_id (one to three
+// default: beside this program), VOSTI_RANDOM_WEIGHTS / --random-weights SEED (the folder needs config.json
+// only; the weights are those of the Python launcher's random-model kind for that seed), VOSTI_STEP_TIMES /
+// --step-times FILE (one line "rows tokens sampled ms" per engine step).  End tokens come from generation_config.json's eos_token_id (one to three
 // ids: python/vosti_kernels/serving_workload.py:78-108); without that file there are none.  It prints
 // MODEL_OUTPUT_TOKEN_IDS=[...] like the reference, or a BENCH batch=... tok_s=... line for prepared requests.
 #include <unistd.h>
@@ -150,6 +152,7 @@ struct Options {
   long page_size = to_int(env_or("VOSTI_PAGE_SIZE", "64"), "VOSTI_PAGE_SIZE");
   long prefix_cache = to_int(env_or("VOSTI_PREFIX_CACHE", "1"), "VOSTI_PREFIX_CACHE");
   std::string lib_dir = env_or("VOSTI_LIB_DIR", "");
+  std::string random_weights = env_or("VOSTI_RANDOM_WEIGHTS", ""), step_times = env_or("VOSTI_STEP_TIMES", "");
 };
 
 Options parse(int argc, char** argv) {
@@ -191,6 +194,8 @@ Options parse(int argc, char** argv) {
     else if (a == "--page-size") o.page_size = to_int(val(), a);
     else if (a == "--prefix-cache") o.prefix_cache = to_int(val(), a);
     else if (a == "--lib-dir") o.lib_dir = val();
+    else if (a == "--random-weights") o.random_weights = val();
+    else if (a == "--step-times") o.step_times = val();
     else throw Usage("unknown option " + a);
   }
   return o;
@@ -226,6 +231,12 @@ int describe(const Options& o) {
   std::sort(names.begin(), names.end());
   names.erase(std::unique(names.begin(), names.end()), names.end());
   for (size_t i = 0; i < names.size(); ++i) out += (i ? ", " : "") + quoted(names[i]);
+  if (!o.random_weights.empty()) {
+    // The seed of every tensor's random stream, as decimal text (they do not fit a double).
+    const uint64_t seed = (uint64_t)to_int(o.random_weights, "--random-weights");
+    out += "], \"tensor_seeds\": [";
+    for (size_t i = 0; i < names.size(); ++i) out += (i ? ", " : "") + quoted(std::to_string(tensor_seed(seed, names[i])));
+  }
   out += "], \"ignored_names\": [";
   for (size_t i = 0; i < spec.ignored_names.size(); ++i) out += (i ? ", " : "") + quoted(spec.ignored_names[i]);
   out += "]";
@@ -273,6 +284,10 @@ int run(int argc, char** argv) {
   eo.prefix_cache = o.prefix_cache == 1;
   eo.max_model_len = (int)o.max_model_len;
   eo.graphs = o.graphs == 1;
+  if (!o.random_weights.empty()) {
+    eo.random_weights = true;
+    eo.random_seed = (uint64_t)to_int(o.random_weights, "--random-weights");
+  }
   {
     // --family names: the model_type of every registered architecture.
     register_builtin_architectures();
@@ -286,6 +301,7 @@ int run(int argc, char** argv) {
     if (architecture != it->second) throw Usage(o.model_path + " holds a " + architecture + ", not a " + o.family + " model");
   }
   Engine engine(eo);
+  engine.record_step_times(!o.step_times.empty());
   std::FILE* trace = nullptr;
   if (!o.step_trace.empty()) {
     trace = std::fopen(o.step_trace.c_str(), "a");
@@ -342,6 +358,14 @@ int run(int argc, char** argv) {
   }
   const Served s = serve(requests, o.seed);
   if (trace) std::fclose(trace);
+  if (!o.step_times.empty()) {
+    std::ofstream f(o.step_times);
+    char buf[96];
+    for (const StepTime& t : engine.step_times()) {
+      std::snprintf(buf, sizeof buf, "%d %d %d %.6f\n", t.rows, t.tokens, t.sampled, t.ms);
+      f << buf;
+    }
+  }
   if (!o.output_tokens.empty()) {
     std::ofstream f(o.output_tokens);
     for (size_t i = 0; i < s.outputs.size(); ++i) f << i << "\t" << id_list(s.outputs[i], ",") << "\n";

@@ -1,6 +1,7 @@
 #include "model.h"
 
 #include <algorithm>
+#include <cmath>
 #include <cstring>
 #include <set>
 #include <sstream>
@@ -210,6 +211,84 @@ void DecoderModel::load_weights(const Checkpoint& ckpt) {
       if (--owners_left[ln.second] == 0) live.erase(it);
     }
     part->load(given);
+  }
+  loaded_ = true;
+}
+
+// BLAKE2b (RFC 7693) with an 8-byte digest and no key, for inputs of any length.
+static uint64_t blake2b_64(const unsigned char* in, size_t len) {
+  static const uint64_t IV[8] = {0x6a09e667f3bcc908ull, 0xbb67ae8584caa73bull, 0x3c6ef372fe94f82bull, 0xa54ff53a5f1d36f1ull,
+                                 0x510e527fade682d1ull, 0x9b05688c2b3e6c1full, 0x1f83d9abfb41bd6bull, 0x5be0cd19137e2179ull};
+  static const unsigned char SIGMA[12][16] = {
+      {0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15}, {14, 10, 4, 8, 9, 15, 13, 6, 1, 12, 0, 2, 11, 7, 5, 3},
+      {11, 8, 12, 0, 5, 2, 15, 13, 10, 14, 3, 6, 7, 1, 9, 4}, {7, 9, 3, 1, 13, 12, 11, 14, 2, 6, 5, 10, 4, 0, 15, 8},
+      {9, 0, 5, 7, 2, 4, 10, 15, 14, 1, 11, 12, 6, 8, 3, 13}, {2, 12, 6, 10, 0, 11, 8, 3, 4, 13, 7, 5, 15, 14, 1, 9},
+      {12, 5, 1, 15, 14, 13, 4, 10, 0, 7, 6, 3, 9, 2, 8, 11}, {13, 11, 7, 14, 12, 1, 3, 9, 5, 0, 15, 4, 8, 6, 2, 10},
+      {6, 15, 14, 9, 11, 3, 0, 8, 12, 2, 13, 7, 1, 4, 10, 5}, {10, 2, 8, 4, 7, 6, 1, 5, 15, 11, 9, 14, 3, 12, 13, 0},
+      {0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15}, {14, 10, 4, 8, 9, 15, 13, 6, 1, 12, 0, 2, 11, 7, 5, 3}};
+  auto rotr = [](uint64_t x, int n) { return (x >> n) | (x << (64 - n)); };
+  uint64_t h[8];
+  for (int i = 0; i < 8; ++i) h[i] = IV[i];
+  h[0] ^= 0x01010000ull ^ 8;            // digest length 8, no key, fanout 1, depth 1
+  size_t done = 0;
+  for (;;) {
+    const bool last = len - done <= 128;
+    const size_t n = last ? len - done : 128;
+    unsigned char block[128] = {0};
+    std::memcpy(block, in + done, n);
+    done += n;
+    uint64_t m[16], v[16];
+    for (int i = 0; i < 16; ++i) {
+      m[i] = 0;
+      for (int b = 7; b >= 0; --b) m[i] = (m[i] << 8) | block[8 * i + b];
+    }
+    for (int i = 0; i < 8; ++i) { v[i] = h[i]; v[i + 8] = IV[i]; }
+    v[12] ^= (uint64_t)done;            // the bytes so far (below 2^64)
+    if (last) v[14] = ~v[14];
+    for (int r = 0; r < 12; ++r) {
+      const unsigned char* s = SIGMA[r];
+      auto G = [&](int a, int b, int c, int d, uint64_t x, uint64_t y) {
+        v[a] = v[a] + v[b] + x; v[d] = rotr(v[d] ^ v[a], 32);
+        v[c] = v[c] + v[d];     v[b] = rotr(v[b] ^ v[c], 24);
+        v[a] = v[a] + v[b] + y; v[d] = rotr(v[d] ^ v[a], 16);
+        v[c] = v[c] + v[d];     v[b] = rotr(v[b] ^ v[c], 63);
+      };
+      G(0, 4, 8, 12, m[s[0]], m[s[1]]);   G(1, 5, 9, 13, m[s[2]], m[s[3]]);
+      G(2, 6, 10, 14, m[s[4]], m[s[5]]);  G(3, 7, 11, 15, m[s[6]], m[s[7]]);
+      G(0, 5, 10, 15, m[s[8]], m[s[9]]);  G(1, 6, 11, 12, m[s[10]], m[s[11]]);
+      G(2, 7, 8, 13, m[s[12]], m[s[13]]); G(3, 4, 9, 14, m[s[14]], m[s[15]]);
+    }
+    for (int i = 0; i < 8; ++i) h[i] ^= v[i] ^ v[i + 8];
+    if (last) break;
+  }
+  return h[0];      // the digest's 8 bytes are h[0] in little-endian order
+}
+
+uint64_t tensor_seed(uint64_t seed, const std::string& name) {
+  const std::string text = std::to_string(seed) + ":" + name;
+  return blake2b_64(reinterpret_cast<const unsigned char*>(text.data()), text.size());
+}
+
+void DecoderModel::random_weights(uint64_t seed) {
+  const auto expected = expected_tensors();
+  std::map<Part*, std::map<std::string, Tensor>> given;
+  for (const auto& e : expected) {
+    const ParamDecl& d = e.second.decl;
+    Tensor t;
+    t.dtype = kernels_.dtype();
+    t.shape = d.shape;
+    t.owner = std::make_shared<DeviceBuffer>(t.bytes());
+    t.data = t.owner->data();
+    // As the kernel takes them: a normal value is a sum of four 16-bit uniforms times std * sqrt(3) / 65536.
+    const float p0 = d.uniform ? (float)d.p0 : (float)(d.p0 * std::sqrt(3.0) / 65536.0);
+    const float p1 = d.uniform ? (float)(d.p1 - d.p0) : 0.f;
+    kernels_.fill_random(t, tensor_seed(seed, e.first), d.uniform ? 1 : 0, p0, p1);
+    for (const auto& o : e.second.owners) given[o.first][o.second] = t;
+  }
+  hip_check(hipStreamSynchronize(kernels_.stream), "random weights");
+  for (Part* part : parts()) {
+    auto it = given.find(part);
+    if (it != given.end()) part->load(it->second);
   }
   loaded_ = true;
 }

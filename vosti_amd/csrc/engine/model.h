@@ -37,6 +37,9 @@ class DecoderModel {
   // loads tensor by tensor: floats become the compute type (a keep_f32 tensor stored in 32-bit stays so),
   // integers int32.
   void load_weights(const Checkpoint& ckpt);
+  // Random weights from a seed, drawn on the GPU: every element is a function of (seed, tensor name, element
+  // index), the values the Python package's random-weights mode stores for the same seed in the compute type.
+  void random_weights(uint64_t seed);
   std::vector<CacheNeed> cache_needs();                     // one per schedule entry (None if it reads another's)
   // ids int32 [T]; caches: one per schedule entry; want_rows int32 [R] -> logits [R, vocab].
   Tensor forward(const Tensor& ids, StepContext& ctx, std::vector<CacheEntry>& caches, const Tensor& want_rows);
@@ -50,6 +53,9 @@ class DecoderModel {
   std::unique_ptr<Head> head_;
   bool loaded_ = false;
 };
+
+// The seed of a tensor's stream: the first 8 bytes, little-endian, of BLAKE2b-64("<seed>:<name>").
+uint64_t tensor_seed(uint64_t seed, const std::string& name);
 
 // Uploads one stored tensor, converted as the rule above says.
 Tensor upload_tensor(const StoredTensor& t, DType compute, bool keep_f32);

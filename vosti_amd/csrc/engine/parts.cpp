@@ -84,7 +84,7 @@ class TokenEmbedding : public Embedding {
 class RMSNorm : public Norm {
  public:
   RMSNorm(const PartSpec& s, Kernels& k) : Norm(k), size_(s.integer("size")), eps_((float)s.number("eps")) {}
-  std::vector<ParamDecl> params() const override { return {{"weight", {size_}, true}}; }
+  std::vector<ParamDecl> params() const override { return {{"weight", {size_}, true, true, 0.9, 1.1}}; }
   void load(std::map<std::string, Tensor>& t) override { weight_ = need(t, "weight"); }
   Tensor forward(const Tensor& x) override { return kernels.rmsnorm(x, weight_, eps_); }
   Tensor forward_add(const Tensor& x, Tensor& residual) override { return kernels.add_rmsnorm(x, residual, weight_, eps_); }

@@ -20,6 +20,9 @@ struct ParamDecl {
   std::string name;               // local name, e.g. "q_proj.weight"
   std::vector<int64_t> shape;
   bool keep_f32 = false;          // a tensor the file stores in 32-bit stays so
+  // Random weights: approximately normal with this standard deviation, or (uniform) in [lo, hi).
+  bool uniform = false;
+  double p0 = 0.02, p1 = 0.0;     // normal: p0 = standard deviation; uniform: p0 = lo, p1 = hi
 };
 
 struct HostArray {

@@ -1,5 +1,6 @@
 from .engine import Engine
+from .native import NativeEngine, NativeEngineError
 from .scheduler import Scheduler
 from .step import ModelRunner, StepEntry
 
-__all__ = ["Engine", "ModelRunner", "Scheduler", "StepEntry"]
+__all__ = ["Engine", "ModelRunner", "NativeEngine", "NativeEngineError", "Scheduler", "StepEntry"]

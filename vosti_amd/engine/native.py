@@ -1,0 +1,150 @@
+"""The native engine behind the Python entry point.
+
+``NativeEngine`` has the face of ``Engine`` (``add_request``, ``step``, ``generate``, ``has_unfinished``) and
+runs plan -> forward -> sample -> commit in C++ (``csrc/engine``, built as ``libvosti_engine.so``): the same
+kernels, cache manager and scheduler, without the Python host code between two steps, which at batch 8 of
+the Qwen3-8B shape is 0.2 of a step's 4.85 ms.  It serves the parts that are built into it; models made of
+parts that are registered from Python run through ``Engine``.  For the same requests and settings both
+produce the same tokens (tests/test_native_engine_gpu.py).
+"""
+from __future__ import annotations
+
+import ctypes
+import json
+from ctypes import c_char_p, c_float, c_int, c_int64, c_uint64, c_void_p
+from pathlib import Path
+
+import numpy as np
+
+from ..kernels import build
+from ..kernels.ops import dtype_name
+from ..sampling import SamplingParams
+
+ABI_VERSION = 1
+_LIB = None
+
+
+class NativeEngineError(RuntimeError):
+    pass
+
+
+def _lib():
+    global _LIB
+    if _LIB is None:
+        import torch  # noqa: F401  (one HIP runtime per process: torch's, loaded first)
+        lib = ctypes.CDLL(str(build.ensure("engine_lib")))
+        lib.ve_abi_version.restype = c_int
+        if lib.ve_abi_version() != ABI_VERSION:
+            raise NativeEngineError(f"libvosti_engine.so has ABI {lib.ve_abi_version()}, expected {ABI_VERSION}; rebuild it")
+        lib.ve_create.restype = c_void_p
+        lib.ve_create.argtypes = [c_char_p, c_char_p, c_char_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_uint64,
+                                  c_char_p, c_int]
+        lib.ve_destroy.argtypes = [c_void_p]
+        lib.ve_add_request.restype = c_int64
+        lib.ve_add_request.argtypes = [c_void_p, c_void_p, c_int, c_int, c_float, c_uint64, c_void_p, c_int, c_int, c_char_p, c_int]
+        lib.ve_step.restype = c_int
+        lib.ve_step.argtypes = [c_void_p, c_void_p, c_int, c_char_p, c_int]
+        lib.ve_has_unfinished.argtypes = [c_void_p]
+        lib.ve_synchronize.argtypes = [c_void_p, c_char_p, c_int]
+        lib.ve_stats.argtypes = [c_void_p, c_void_p]
+        lib.ve_cache_check.argtypes = [c_void_p, c_char_p, c_int]
+        _LIB = lib
+    return _LIB
+
+
+class NativeEngine:
+    def __init__(self, model_dir: str | Path, *, dtype="bfloat16", num_pages: int = 32, page_size: int = 64, max_num_seqs: int = 8,
+                 max_num_batched_tokens: int = 4096, enable_prefix_cache: bool = True, max_model_len: int | None = None,
+                 graphs: bool = False, random_weights_seed: int | None = None):
+        """The arguments of ``Engine``; ``model_dir`` must be a folder (config.json and safetensors).  With
+        ``random_weights_seed`` the folder needs config.json only and the weights are drawn on the GPU from
+        that seed (the values ``write_random_model`` stores for it)."""
+        self._lib = _lib()
+        name = dtype_name(dtype)
+        kernels = build.ensure(name)              # the engine loads the kernel library of its precision from here
+        self._err = ctypes.create_string_buffer(4096)
+        self.max_num_seqs = max_num_seqs
+        self._h = self._lib.ve_create(str(model_dir).encode(), str(kernels.parent).encode(), name.encode(), num_pages, page_size,
+                                      max_num_seqs, max_num_batched_tokens, 1 if enable_prefix_cache else 0, max_model_len or 0,
+                                      1 if graphs else 0, 0 if random_weights_seed is None else 1,
+                                      (random_weights_seed or 0) & (2**64 - 1), self._err, len(self._err))
+        if not self._h:
+            raise NativeEngineError(self._err.value.decode(errors="replace"))
+        self._out = np.empty((max_num_seqs + 1, 2), dtype=np.int64)
+        self.steps = 0
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h:
+            self._lib.ve_destroy(h)
+
+    def _fail(self):
+        raise NativeEngineError(self._err.value.decode(errors="replace"))
+
+    # ------------------------------------------------------------- requests
+    def add_request(self, prompt_ids: list[int], params: SamplingParams | None = None) -> int:
+        params = params or SamplingParams()
+        prompt = np.asarray(prompt_ids, dtype=np.int32)
+        eos = np.asarray(params.eos_token_ids, dtype=np.int32)
+        rid = self._lib.ve_add_request(self._h, prompt.ctypes.data, len(prompt), params.max_tokens, params.temperature,
+                                       params.seed & (2**64 - 1), eos.ctypes.data if len(eos) else None, len(eos),
+                                       1 if params.ignore_eos else 0, self._err, len(self._err))
+        if rid < 0:
+            raise ValueError(self._err.value.decode(errors="replace"))
+        return rid
+
+    def has_unfinished(self) -> bool:
+        return bool(self._lib.ve_has_unfinished(self._h))
+
+    # ----------------------------------------------------------------- step
+    def step(self) -> dict[int, int]:
+        """One engine step.  Returns {request id: emitted token} for the requests that emitted one."""
+        n = self._lib.ve_step(self._h, self._out.ctypes.data, len(self._out), self._err, len(self._err))
+        if n < 0:
+            self._fail()
+        self.steps += 1
+        return {int(r): int(t) for r, t in self._out[:n]}
+
+    def synchronize(self) -> None:
+        if self._lib.ve_synchronize(self._h, self._err, len(self._err)) != 0:
+            self._fail()
+
+    def stats(self) -> dict:
+        out = np.zeros(10, dtype=np.int64)
+        self._lib.ve_stats(self._h, out.ctypes.data)
+        names = ("eager", "captured", "replayed", "evicted")
+        return {"graph_stats": dict(zip(names, map(int, out[:4]))), "prefix_hit_requests": int(out[4]), "prefix_hits": int(out[5]),
+                "preemptions": int(out[6]), "cache_requests": int(out[7]), "vocab_size": int(out[8]), "max_positions": int(out[9])}
+
+    def cache_check(self) -> str:
+        buf = ctypes.create_string_buffer(1024)
+        self._lib.ve_cache_check(self._h, buf, len(buf))
+        return buf.value.decode()
+
+    # ------------------------------------------------------------- generate
+    def generate(self, prompts: list[list[int]], params: SamplingParams | list[SamplingParams] | None = None,
+                 arrival_steps: list[int] | None = None, trace=None) -> list[list[int]]:
+        """As ``Engine.generate``: ``arrival_steps[i]`` delays prompt i until that engine step; ``trace`` gets one
+        JSON line per step (without the ids scheduled, which stay inside the native engine)."""
+        if params is None or isinstance(params, SamplingParams):
+            params = [params or SamplingParams()] * len(prompts)
+        arrival_steps = arrival_steps or [0] * len(prompts)
+        pending = sorted(range(len(prompts)), key=lambda i: (arrival_steps[i], i))
+        ids: dict[int, int] = {}
+        outputs: list[list[int]] = [[] for _ in prompts]
+        step = 0
+        while pending or self.has_unfinished():
+            arrived = []
+            while pending and arrival_steps[pending[0]] <= step:
+                i = pending.pop(0)
+                ids[self.add_request(prompts[i], params[i])] = i
+                arrived.append(i)
+            emitted = self.step()
+            for rid, tok in emitted.items():
+                if rid in ids:
+                    outputs[ids[rid]].append(tok)
+            if trace is not None:
+                trace.write(json.dumps({"step": step, "arrived": arrived,
+                                        "emitted": {str(ids.get(r, r)): t for r, t in emitted.items()}}) + "\n")
+            step += 1
+        return outputs

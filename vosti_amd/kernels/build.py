@@ -7,7 +7,9 @@ Three shared libraries and one program are built from ``vosti_amd/csrc``:
 * ``libvosti_host.so``: the cache manager and the scheduler (g++, no GPU code);
 * ``vosti_engine``: the native engine and its command line (``csrc/engine`` with
   the cache manager and the scheduler compiled in; g++ against the HIP runtime;
-  it loads the kernel library of the chosen precision from its own folder).
+  it loads the kernel library of the chosen precision from its own folder), and
+  ``libvosti_engine.so``: the same engine behind a C interface (``capi.cpp``
+  instead of ``main.cpp``), which ``vosti_amd.engine.NativeEngine`` drives.
 
 A library is rebuilt when the hash of its sources, headers and flags differs
 from the one recorded beside it.  ``ensure()``
@@ -67,7 +69,9 @@ def build_dir() -> Path:
 
 
 def _file_name(name: str) -> str:
-    return "vosti_engine" if name == "engine" else f"libvosti_{name}.so"
+    if name == "engine":
+        return "vosti_engine"
+    return "libvosti_engine.so" if name == "engine_lib" else f"libvosti_{name}.so"
 
 
 def lib_path(name: str) -> Path:
@@ -86,9 +90,10 @@ def _sources(name: str) -> tuple[list[Path], list[Path]]:
     host = CSRC / "host"
     if name == "host":
         return sorted(host.glob("*.cpp")), sorted(host.glob("*.h"))
-    if name == "engine":
+    if name in ("engine", "engine_lib"):
         engine = CSRC / "engine"
-        return (sorted(engine.glob("*.cpp")) + [host / "cache_manager.cpp", host / "scheduler.cpp"],
+        face = "capi.cpp" if name == "engine" else "main.cpp"       # the file of the other face is left out
+        return ([p for p in sorted(engine.glob("*.cpp")) if p.name != face] + [host / "cache_manager.cpp", host / "scheduler.cpp"],
                 sorted(engine.glob("*.h")) + sorted(host.glob("*.h")))
     return sorted(CSRC.glob("*.hip")), sorted(CSRC.glob("*.h"))
 
@@ -96,7 +101,7 @@ def _sources(name: str) -> tuple[list[Path], list[Path]]:
 def _flags(name: str) -> list[str]:
     if name == "host":
         return HOST_FLAGS
-    if name == "engine":
+    if name in ("engine", "engine_lib"):
         return HOST_FLAGS + ["-I", str(rocm_root() / "include")]
     return HIPCC_FLAGS + [f"-D{GPU_LIBS[name]}"]
 
@@ -131,13 +136,13 @@ def _run(cmd: list[str], what: str) -> None:
 
 
 def build(name: str, verbose: bool = True) -> Path:
-    """Compile library ``name`` ('bf16', 'f32' or 'host') or the program 'engine' unconditionally."""
+    """Compile library ``name`` ('bf16', 'f32', 'host', 'engine_lib') or the program 'engine' unconditionally."""
     srcs, _ = _sources(name)
     if not srcs:
         raise RuntimeError(f"no sources for library {name!r} under {CSRC}")
     obj_dir = build_dir() / name
     obj_dir.mkdir(parents=True, exist_ok=True)
-    if name in ("host", "engine"):
+    if name in ("host", "engine", "engine_lib"):
         compiler = _find("g++", "/usr/bin/g++")
     else:
         compiler = _find("hipcc", "/opt/rocm/bin/hipcc")
@@ -166,7 +171,10 @@ def build(name: str, verbose: bool = True) -> Path:
         return out
     tmp = out.with_suffix(f".tmp{os.getpid()}.so")
     link = [compiler, "-shared", "-fPIC", "-o", str(tmp), *map(str, objs)]
-    if name != "host":
+    if name == "engine_lib":
+        rocm_lib = str(rocm_root() / "lib")
+        link += ["-L", rocm_lib, "-lamdhip64", "-ldl", f"-Wl,-rpath,{rocm_lib}"]
+    elif name != "host":
         link.insert(1, f"--offload-arch={GPU_ARCH}")
     _run(link, out.name)
     # A kernel whose host-side stub the compiler left out shows as an undefined symbol only when the
@@ -193,7 +201,7 @@ def ensure(name: str, verbose: bool = True) -> Path:
 
 
 def build_all(verbose: bool = True) -> None:
-    for name in ("host", "engine", "bf16", "f32"):
+    for name in ("host", "engine", "engine_lib", "bf16", "f32"):
         build(name, verbose)
 
 
