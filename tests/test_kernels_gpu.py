@@ -34,7 +34,7 @@ def rand(shape, dtype, seed, scale=1.0):
                                    (65, 130, 520), (130, 96, 1032), (300, 520, 2056), (8, 40, 4104),
                                    (8, 4100, 1024), (3, 72, 512), (33, 200, 1536), (64, 4096, 4608), (17, 90, 5120),
                                    (40, 6200, 1024), (64, 6144, 512), (23, 24, 2048), (48, 24700, 512), (20, 24576, 1024), (31, 6200, 4096), (17, 100, 1536), (9, 130, 12288), (16, 72, 8704), (2, 40, 5120), (100, 200, 1024), (65, 4100, 512), (130, 96, 1536),
-                                   (250, 8200, 512), (129, 300, 4608), (300, 8400, 128), (700, 9000, 64)])
+                                   (250, 8200, 512), (129, 300, 4608), (300, 8400, 128), (700, 9000, 64), (300, 520, 2048), (520, 1000, 4096)])
 def test_gemm(dtype, M, N, K):
     k = kern(dtype)
     a, w = rand((M, K), dtype, 1), rand((N, K), dtype, 2, 0.1)

@@ -34,6 +34,8 @@
 #define KC_SLABS (KC / VK_SLAB)       // 16 (bfloat16) or 32 (float)
 #define SK_WAVES 8
 
+static int device_cus();      // compute units of the current device (defined with the host code below)
+
 __device__ __forceinline__ void store_out4(elem_t* out, int64_t ldo, int m, int n, int M, int N, f32x4 v,
                                            bool vec_ok) {
   if (m >= M || n >= N) return;
@@ -535,7 +537,19 @@ __device__ __forceinline__ unsigned lds_offset_of(const unsigned char* p) {
 
 // FNW: 16-row weight fragments per wave, 4 (a workgroup takes 128 weight rows) or 2 (64: twice the
 // workgroups, for grids that would leave compute units with one workgroup or none).
-template <int S, bool WHOLE, bool SWIGLU, int FNW = 4>
+// One 4-byte load per lane whose value nobody reads: it brings the lane's 128-byte line into the second-level
+// cache ahead of the LDS-direct load that will want it.  `keep` is one register that every such load writes
+// (in order, so they may overlap) and that stays allocated to the end of the kernel.
+__device__ __forceinline__ void pipe_touch_line(const unsigned char* sbase, unsigned voff, unsigned& keep) {
+  asm volatile("global_load_dword %0, %1, %2 sc1" : "+v"(keep) : "v"(voff), "s"(sbase) : "memory");
+}
+template <int N_>
+__device__ __forceinline__ void wait_vmcnt_n() {             // vmcnt(N_), N_ below 64; the other counters at their maxima
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (N_ & 0xF) | ((N_ >> 4) << 14));
+}
+
+// PFD > 0: every wave touches, PFD tiles ahead, the 64 rows of the workgroup's tiles that are its share.
+template <int S, bool WHOLE, bool SWIGLU, int FNW = 4, int PFD = 0>
 __global__ __launch_bounds__(256, 2) void gemm_pipe_kernel(elem_t* __restrict__ out, const elem_t* __restrict__ act,
                                                         const elem_t* __restrict__ w, int M, int N, int K,
                                                         int64_t lda, int64_t ldo, int out_vec_ok, int band_w) {
@@ -600,6 +614,24 @@ __global__ __launch_bounds__(256, 2) void gemm_pipe_kernel(elem_t* __restrict__ 
     for (int j = 0; j < 4; ++j) pipe_load_to_lds16_sv(abase + kb, offa[j], base + W_BYTES + (wave * 4 + j) * 8 * T_ROWB);
   };
 
+  // The lines a wave touches ahead: row wave * 64 + lane of the workgroup's weight rows followed by its
+  // activation rows (a wave's 64 rows are all weights, all up rows, or all activations).
+  static_assert(PFD == 0 || S == 2, "the touch-ahead counts its loads for two stages");
+  unsigned pf_off = 0, pf_keep = 0;
+  const unsigned char* pf_base = wbase;
+  if (PFD > 0) {
+    const int r = wave * 64 + lane;
+    if (wave * 64 < BN) {
+      const bool up = SWIGLU && wave * 64 >= 64;
+      const int local = up ? r - 64 : r;
+      pf_base = up ? ubase : wbase;
+      pf_off = (unsigned)((int64_t)(min(n_blk + local, N - 1) - min(n_blk, N - 1)) * K * (int64_t)sizeof(elem_t));
+    } else {
+      pf_base = abase;
+      pf_off = (unsigned)((int64_t)(min(m_blk + min(r - BN, 127), M - 1) - min(m_blk, M - 1)) * lda * (int64_t)sizeof(elem_t));
+    }
+  }
+
   f32x4 acc[FNW][4], total[FNW][4];
 #pragma unroll
   for (int i = 0; i < FNW; ++i)
@@ -615,10 +647,16 @@ __global__ __launch_bounds__(256, 2) void gemm_pipe_kernel(elem_t* __restrict__ 
 
   auto step = [&](int kt) {
     // Tile kt has landed once at most the loads of the tiles after it are outstanding (FNW + 4 per tile and wave).
-    const int later = min(S - 2, ntiles - 1 - kt);
-    wait_vmcnt((FNW + 4) * later);
+    if (PFD > 0) {
+      if (kt == 0) wait_vmcnt_n<0>(); else wait_vmcnt_n<1>();      // the one touch that was issued behind tile kt's loads may still fly
+    } else {
+      const int later = min(S - 2, ntiles - 1 - kt);
+      wait_vmcnt((FNW + 4) * later);
+    }
     __syncthreads();       // every wave's part of tile kt is there; everyone is done with tile kt-1's buffer
     if (kt + S - 1 < ntiles) issue(kt + S - 1);
+    if (PFD > 0)           // always one, so that the count above holds: beyond the end the last tile again
+      pipe_touch_line(pf_base + (int64_t)min(kt + PFD, ntiles - 1) * 2 * VK_SLAB * (int64_t)sizeof(elem_t), pf_off, pf_keep);
     const unsigned char* base = lds + (kt % S) * STAGE_BYTES;
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
@@ -672,6 +710,10 @@ __global__ __launch_bounds__(256, 2) void gemm_pipe_kernel(elem_t* __restrict__ 
     }
   }
 
+  if (PFD > 0) {
+    wait_vmcnt_n<0>();                                        // the last touches
+    asm volatile("" : : "v"(pf_keep));                        // the register was theirs until here
+  }
   if constexpr (SWIGLU) {
     // The two waves of a row block split the 64 output columns: the gate wave keeps columns 0..31 and
     // gets their up values, the up wave keeps columns 32..63 and gets their gate values.
@@ -733,6 +775,21 @@ static int launch_pipe(elem_t* out, const elem_t* act, const elem_t* w, int M, i
   dim3 grid((N + BN - 1) / BN, (M + 127) / 128);
   VK_REQUIRE(grid.y <= 65535, "gemm: too many rows (%d)", M);
   const int band_w = (pipe_band_blocks > 0 && grid.y > 1 && (int)grid.x > pipe_band_blocks) ? pipe_band_blocks : (int)grid.x;
+  if constexpr (S == 2) {
+    // No more workgroups than compute units: each waits for its own loads with nothing to run meanwhile, and
+    // touching the lines four tiles ahead brings them into the second-level cache in time (300 rows, 4,096 x
+    // 12,288: 146 -> 112 us).  With more workgroups the touches cost more than they bring: the path from
+    // that cache into LDS is as busy as the MFMA unit (2,048 rows: 1,057 -> 660 TFLOP/s).
+    if (K % KC == 0 && (int64_t)grid.x * grid.y <= device_cus()) {
+      static bool touched = false;
+      if (!touched) {
+        (void)hipFuncSetAttribute((const void*)gemm_pipe_kernel<S, true, SWIGLU, FNW, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        touched = true;
+      }
+      gemm_pipe_kernel<S, true, SWIGLU, FNW, 4><<<grid, 256, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok, band_w);
+      return vk_check_launch("gemm_pipe");
+    }
+  }
   if (K % KC == 0) gemm_pipe_kernel<S, true, SWIGLU, FNW><<<grid, 256, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok, band_w);
   else gemm_pipe_kernel<S, false, SWIGLU, FNW><<<grid, 256, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok, band_w);
   return vk_check_launch("gemm_pipe");
@@ -951,8 +1008,6 @@ static int launch_mid(elem_t* out, const elem_t* act, const elem_t* w, int M, in
   gemm_mid_kernel<MT, KH, SWIGLU, GT><<<grid, 512, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok);
   return vk_check_launch("gemm_mid");
 }
-
-static int device_cus();
 
 // ---------------------------------------------------------------- split
 // 17 to 64 rows and few weight rows: the kernels above give such a product a workgroup or less per compute
