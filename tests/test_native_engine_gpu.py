@@ -183,6 +183,26 @@ def test_native_engine_from_python(tiny_dirs, dtype_name, graphs):
         NativeEngine("/nonexistent", dtype=dtype_name)
 
 
+def test_python_launcher_with_the_native_engine(tiny_dirs, tmp_path):
+    """--engine native of the Python launcher prints what --engine python prints (but for the wall time)."""
+    import sys
+    from conftest import ROOT
+    ps = prompts("B", [30, 30, 12], seed=4)
+    ps[1] = ps[0][:24] + ps[1][24:]                    # shares three pages of 8 with the first
+    tsv(tmp_path / "reqs.tsv", [(6, p, a) for p, a in zip(ps, [0, 2, 2])])
+    lines = {}
+    for which in ("python", "native"):
+        r = subprocess.run([sys.executable, "-m", "vosti_amd.launch", "--kind", "engine", "--family", "qwen3", "--", "--engine", which,
+                            "--model-path", str(tiny_dirs["B"]), "--bench-input", str(tmp_path / "reqs.tsv"), "--page-size", "8",
+                            "--num-blocks", "24", "--graphs", "1", "--output-tokens", str(tmp_path / f"{which}.tsv")],
+                           env=dict(os.environ, PYTHONPATH=str(ROOT)), capture_output=True, text=True, timeout=110)
+        assert r.returncode == 0, r.stderr[-2000:]
+        lines[which] = [l.split(" wall_s=")[0] for l in r.stdout.splitlines() if l.split(" ")[0] in ("BENCH", "CACHE_STATS", "GRAPH_STATS")]
+    assert lines["native"] == lines["python"] and len(lines["native"]) == 3
+    assert (tmp_path / "native.tsv").read_text() == (tmp_path / "python.tsv").read_text()
+    assert '"reused_prefix_blocks":3' in lines["native"][1]
+
+
 def test_one_error_for_weights_that_do_not_fit(program, tiny_dirs, tmp_path):
     d = tmp_path / "model"
     shutil.copytree(tiny_dirs["B"], d)

@@ -30,7 +30,10 @@ here; each also has a command-line option, which wins:
 
 Options without a counterpart in the reference: VOSTI_DTYPE / --dtype (bfloat16,
 float32), VOSTI_TEMPERATURE / --temperature, VOSTI_SEED / --seed,
-VOSTI_PAGE_SIZE / --page-size, VOSTI_PREFIX_CACHE / --prefix-cache (0, 1).
+VOSTI_PAGE_SIZE / --page-size, VOSTI_PREFIX_CACHE / --prefix-cache (0, 1),
+VOSTI_ENGINE / --engine (python, native: the same engine driven from C++,
+``vosti_amd.engine.NativeEngine``; the whole launcher as a native program is
+``bin/vosti_engine``).
 End tokens come from generation_config.json's ``eos_token_id`` (one to three
 ids: python/vosti_kernels/serving_workload.py:78-108); without that file there
 are none.  It prints ``MODEL_OUTPUT_TOKEN_IDS=[...]`` like the reference, or a
@@ -81,6 +84,7 @@ def engine_parser() -> argparse.ArgumentParser:
     p.add_argument("--seed", type=int, default=int(_env("VOSTI_SEED", 0)))
     p.add_argument("--page-size", type=int, default=int(_env("VOSTI_PAGE_SIZE", 64)))
     p.add_argument("--prefix-cache", type=int, default=int(_env("VOSTI_PREFIX_CACHE", 1)), choices=[0, 1])
+    p.add_argument("--engine", default=_env("VOSTI_ENGINE", "python"), choices=["python", "native"])
     return p
 
 
@@ -204,6 +208,10 @@ def run_engine(argv: list[str], family: str) -> int:
         requests = [(args.max_tokens, parse_ids(args.prompt_ids), 0)]
     warmup = parse_prepared(args.bench_warmup_input) if args.bench_input and args.bench_warmup_input else []
     eos = eos_ids(args.model_path)
+    if args.engine == "native":
+        if args.bench_calls or os.environ.get("VOSTI_LOGITS_DIGEST") or os.environ.get("VOSTI_LOGITS_OBSERVER_DIR"):
+            raise SystemExit("--engine native serves neither the multi-call driver nor the logits observers; use --engine python")
+        from .engine import NativeEngine as Engine
     engine = Engine(args.model_path, dtype=args.dtype, num_pages=args.num_blocks, page_size=args.page_size,
                     max_num_seqs=args.max_seqs or max(len(requests), len(warmup), 1 if not args.bench_calls else 8),
                     max_num_batched_tokens=args.max_batched_tokens, enable_prefix_cache=bool(args.prefix_cache),
@@ -213,17 +221,24 @@ def run_engine(argv: list[str], family: str) -> int:
     trace = open(args.step_trace, "a") if args.step_trace else None
     import torch
 
+    def cache_counters():
+        if args.engine == "native":
+            st = engine.stats()
+            return st["prefix_hit_requests"], st["prefix_hits"]
+        return engine.cache.prefix_hit_requests(), engine.cache.prefix_hits()
+
     def serve(reqs, first_seed):
         """(outputs, wall seconds, cache statistics of this workload alone)."""
         params = [SamplingParams(max_tokens=m, temperature=args.temperature, seed=first_seed + i, eos_token_ids=eos,
                                  ignore_eos=args.ignore_eos) for i, (m, _, _) in enumerate(reqs)]
-        before = (engine.cache.prefix_hit_requests(), engine.cache.prefix_hits())
+        before = cache_counters()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         outs = engine.generate([ids for _, ids, _ in reqs], params, [a for _, _, a in reqs], trace=trace)
         wall = time.perf_counter() - t0
-        stats = {"admitted_requests": len(reqs), "requests_with_reuse": engine.cache.prefix_hit_requests() - before[0],
-                 "reused_prefix_blocks": engine.cache.prefix_hits() - before[1]}
+        after = cache_counters()
+        stats = {"admitted_requests": len(reqs), "requests_with_reuse": after[0] - before[0],
+                 "reused_prefix_blocks": after[1] - before[1]}
         return outs, wall, stats
 
     def line(tag, reqs, outs, wall, rate):
@@ -244,12 +259,13 @@ def run_engine(argv: list[str], family: str) -> int:
         Path(args.output_tokens).write_text("".join(f"{i}\t{','.join(map(str, o))}\n" for i, o in enumerate(outputs)))
     if args.bench_input:
         print(line("BENCH", requests, outputs, wall, rate=True))
-        stats["preemptions"] = engine.scheduler.preemptions()
+        stats["preemptions"] = engine.stats()["preemptions"] if args.engine == "native" else engine.scheduler.preemptions()
         print("CACHE_STATS " + json.dumps(stats, separators=(",", ":")))
     else:
         print(f"MODEL_OUTPUT_TOKEN_IDS={outputs[0]}")
     if args.graphs:
-        print("GRAPH_STATS " + json.dumps(engine.runner.graph_stats, separators=(",", ":")))
+        graph_stats = engine.stats()["graph_stats"] if args.engine == "native" else engine.runner.graph_stats
+        print("GRAPH_STATS " + json.dumps(graph_stats, separators=(",", ":")))
     return 0
 
 
