@@ -1144,6 +1144,65 @@ static int device_cus() {
   return cus;
 }
 
+// Which kernel computes a product (speed only: all give the same bits).  Every threshold is a count of
+// workgroups against the device's compute units (cus), or a count of 16-row activation tiles, or whether a
+// wave's share of K fits its registers; none is a model's size.  With the workgroups a kernel would start:
+//   wg16  = ceil(N / 16)   the streaming kernels (one 16-row weight tile a workgroup; two with kernel 7)
+//   wg32, wg64, wg128      the kernel that shares activations through LDS (32, 64 or 128 weight rows a workgroup)
+//   k_resident             K <= 8 chunks: each of a workgroup's 8 waves has one chunk, whose activations stay in registers
+//
+//   rows     condition                                         kernel
+//   1..16                                                      1   streaming
+//   17..32   16-bit, K whole chunks, k_resident,               11  streaming, both activation tiles of a wave's chunk in
+//            wg16 >= 1.5 cus                                       registers (32 rows, 24576 x 4096: 53 -> 44 us)
+//   17..64   K whole chunks:
+//              wg128 >= 0.75 cus                               10  128 weight rows a workgroup: the activations that every
+//                                                                  workgroup reads are half the weight bytes (64 rows, 51200 x
+//                                                                  5120: 158 -> 127 us)
+//              wg64 >= 0.5 cus                                 8   64 weight rows a workgroup
+//              rows > 32, wg32 <= 0.5 cus, and rows > 40 or    12  so few weight rows that workgroups of 32 leave half the units
+//                not k_resident                                    idle: two blocks of 32 rows side by side (64 rows, 4096 x
+//                                                                  12288: 55 -> 45 us)
+//              rows > 40                                       9   32 weight rows a workgroup
+//              k_resident or wg16 <= cus                       7 / 1  streaming, two weight tiles a workgroup from wg16 >= 1.5 cus
+//              else                                            9   the streaming kernel would need a second pass for a few tiles
+//                                                                  (32 rows, 5120 x 17408: 111 -> 65 us)
+//   17..64   K not in whole chunks                             2 (rows > 32 and wg128 >= 0.5 cus), else 7 / 1 as above
+//   65..256  K whole chunks, wg128 < 0.5 cus:                      the tile kernel would have a workgroup or less per unit, each
+//                                                                  walking all of K alone (4096 x 12288: 170 us at any of these
+//                                                                  rows); the LDS-sharing kernel in blocks of 64 rows fills the
+//                                                                  chip (100 rows: 51 us, 200 rows: 82 us)
+//              wg64 >= 0.5 cus                                 8 up to three blocks, else 2
+//              two blocks                                      9 (wg32 <= 0.5 cus) or 8
+//              else                                            2 (k_resident and wg16 >= 1.5 cus) or 8
+//   more                                                       2   the pipelined tile kernel
+// With a workspace the products of 17 to 64 rows that vk_gemm_split_preferred names go through chunk sums
+// instead (the caller's choice: vk_gemm_split).
+static int choose_gemm_kernel(int M, int N, int K) {
+  const int cus = device_cus();
+  const int wg16 = (N + 15) / 16, wg32 = (N + 31) / 32, wg64 = (N + 63) / 64, wg128 = (N + 127) / 128;
+  const bool whole = K % KC == 0, k_resident = K <= SK_WAVES * KC;
+  const bool many16 = 2 * wg16 >= 3 * cus;
+  if (M <= 16) return 1;
+  if (M <= 32 && whole && k_resident && many16 && sizeof(elem_t) == 2) return 11;
+  if (M <= 64 && whole) {
+    if (4 * wg128 >= 3 * cus) return 10;
+    if (2 * wg64 >= cus) return 8;
+    if (M > 32 && 2 * wg32 <= cus && (M > 40 || !k_resident)) return 12;
+    if (M > 40) return 9;
+    if (k_resident || wg16 <= cus) return many16 ? 7 : 1;
+    return 9;
+  }
+  if (M <= 64) return (2 * wg128 >= cus && M > 32) ? 2 : (many16 ? 7 : 1);
+  if (M <= 256 && whole && 2 * wg128 < cus) {
+    const int blocks = (M + 63) / 64;
+    if (2 * wg64 >= cus) return blocks <= 3 ? 8 : 2;
+    if (blocks == 2) return 2 * wg32 <= cus ? 9 : 8;
+    return (k_resident && many16) ? 2 : 8;
+  }
+  return 2;
+}
+
 extern "C" {
 
 // kernel: 0 = choose by size, 1 = skinny (M <= 64), 2 = tiled (pipelined if K allows), 3 = tiled through
@@ -1163,42 +1222,8 @@ int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K
   VK_REQUIRE(kernel >= 0 && kernel <= 13, "gemm: unknown kernel %d", kernel);
   if (M == 0) return 0;
   const int vec_ok = (ldo % 4 == 0) && ((uintptr_t)out % 16 == 0);
-  // Measured on Qwen3-8B shapes (MI355X).  Up to 16 rows: the streaming kernel.  17 to 32 rows of 16-bit
-  // elements with K up to 4096 and 6144 weight rows or more: the streaming kernel with both activation
-  // tiles of a wave's chunk in registers (32 rows, 24576 x 4096: 53 -> 44 us).  Else 17 to 64 rows with K in
-  // whole chunks: the kernel that shares activations through LDS: 128 weight rows per workgroup from
-  // 24576 weight rows on (the activations that every workgroup reads are then half the weight bytes:
-  // 64 rows, 51200 x 5120: 158 -> 127 us), 64 from 8192 on; with fewer, 32 weight rows from 41 rows on, or
-  // when K is over 4096 and there are more 16-row weight tiles than compute units, so that the streaming
-  // kernel would need a second pass for a few of them (32 rows, 5120 x 17408: 111 -> 65 us); and below
-  // that the streaming kernel, with two weight tiles per workgroup from 6144 weight rows on.  More
-  // rows: the pipelined tile kernel.
   const bool by_size = kernel == 0;
-  if (kernel == 0) {
-    if (M <= 16) kernel = 1;
-    else if (M <= 32 && K % KC == 0 && K <= SK_WAVES * KC && N >= 6144 && sizeof(elem_t) == 2) kernel = 11;
-    else if (M <= 64 && K % KC == 0) {
-      if (N >= 24576) kernel = 10;
-      else if (N >= 8192) kernel = 8;
-      // So few weight rows that workgroups of 32 of them leave half the compute units idle: two blocks
-      // of 32 rows each, side by side (64 rows, 4096 x 12288: 55 -> 45 us).
-      else if (M > 32 && 2 * ((N + 31) / 32) <= device_cus() && (M > 40 || K > SK_WAVES * KC)) kernel = 12;
-      else if (M > 40) kernel = 9;
-      else if (K <= SK_WAVES * KC || (N + 15) / 16 <= device_cus()) kernel = N >= 6144 ? 7 : 1;
-      else kernel = 9;
-    }
-    else if (M <= 64) kernel = (N >= 16384 && M > 32) ? 2 : (N >= 6144 ? 7 : 1);
-    else if (M <= 256 && K % KC == 0 && N < 16384) {
-      // 65 to 256 rows and few weight rows: the tile kernel would have a workgroup or less per compute
-      // unit, each walking all of K on its own (4096 x 12288 takes it 170 us at any of these sizes); the
-      // kernel above in blocks of 64 rows fills the chip (100 rows: 51 us, 200 rows: 82 us).
-      const int blocks = (M + 63) / 64;
-      if (N >= 8192) kernel = blocks <= 3 ? 8 : 2;
-      else if (blocks == 2) kernel = N <= 4096 ? 9 : 8;
-      else kernel = (K <= SK_WAVES * KC && N >= 6144) ? 2 : 8;
-    }
-    else kernel = 2;
-  }
+  if (kernel == 0) kernel = choose_gemm_kernel(M, N, K);
   if (kernel == 12) {      // 32 weight rows per workgroup, four chunks in work, blocks of 32 rows
     VK_REQUIRE(M > 16 && M <= 512 && K % KC == 0, "gemm: the mid kernel takes 17 to 512 rows and K a multiple of %d", KC);
     return launch_mid<2, 4>(out, act, w, M, N, K, lda, ldo, vec_ok, st);
@@ -1385,14 +1410,17 @@ int64_t vk_gemm_split_floats(int M, int rows, int K, int swiglu) {
 #endif
 }
 
-// 1 if the route through chunk sums is the faster one for these sizes (measured on Qwen3-8B shapes, MI355X,
-// 64 rows: 4096 x 12288 45 -> 32 us, 6144 x 4096 20.6 -> 18.2 us, 4096 x 4096 16.0 -> 13.8 us; 32 rows:
-// 41 -> 27, 17.8 -> 14.7, 13.4 -> 11.7 us).  Not with the activation folded in (24576 x 4096: 60 -> 62 us), not
-// for small matrices (1000 x 1024 at 32 rows: 4.8 -> 6.5 us), and not for very many weight rows, where the
-// other kernels have workgroups enough and the chunk sums would be a large share of the traffic.
+// 1 if the route through chunk sums is the faster one for these sizes (measured with 4096 to 6144 weight rows
+// and K of 4096 and 12288 on an MI355X, 64 rows: 4096 x 12288 45 -> 32 us, 6144 x 4096 20.6 -> 18.2 us, 4096 x
+// 4096 16.0 -> 13.8 us; 32 rows: 41 -> 27, 17.8 -> 14.7, 13.4 -> 11.7 us).  Not with the activation folded in (24576
+// x 4096: 60 -> 62 us), not for matrices of less than 64 KB per compute unit (1000 x 1024 at 32 rows: 4.8 -> 6.5
+// us), and not where workgroups of 128 weight rows are a quarter of the compute units or more: the other
+// kernels then have workgroups enough, and the chunk sums would be a large share of the traffic.
 int vk_gemm_split_preferred(int M, int rows, int K, int swiglu) {
   if (swiglu || vk_gemm_split_floats(M, rows, K, swiglu) == 0) return 0;
-  return (int64_t)rows * K >= ((int64_t)1 << 23) && rows <= 8192;
+  const int cus = device_cus();
+  const int64_t bytes = (int64_t)rows * K * (int64_t)sizeof(elem_t);
+  return bytes >= (int64_t)cus * 65536 && 4 * ((rows + 127) / 128) <= cus;
 }
 
 // out = act w^T (swiglu 0: w [rows, K], out [M, rows]) or silu(act w_gate^T) * (act w_up^T) (swiglu 1:
