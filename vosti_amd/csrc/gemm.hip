@@ -718,14 +718,16 @@ __global__ __launch_bounds__(256, 2) void gemm_pipe_kernel(elem_t* __restrict__ 
     // The two waves of a row block split the 64 output columns: the gate wave keeps columns 0..31 and
     // gets their up values, the up wave keeps columns 32..63 and gets their gate values.
     __syncthreads();            // the last tile has been read: LDS is free
-    f32x4* ex = reinterpret_cast<f32x4*>(lds);      // [128 rows][16 groups of 4 columns]
+    // [128 rows][16 groups of 4 columns]; a row's group g lies at place g ^ (row % 16), so that the 16 rows a
+    // wave touches at once (256 bytes apart: the same banks) spread over all banks.
+    f32x4* ex = reinterpret_cast<f32x4*>(lds);
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         f32x4& v = total[i][j];
         v.x = round_to_elem(v.x); v.y = round_to_elem(v.y); v.z = round_to_elem(v.z); v.w = round_to_elem(v.w);
-        if ((i < 2) == (wn == 1)) ex[(wm * 64 + j * 16 + r16) * 16 + i * 4 + kg] = v;    // what the other wave needs
+        if ((i < 2) == (wn == 1)) ex[(wm * 64 + j * 16 + r16) * 16 + ((i * 4 + kg) ^ r16)] = v;    // what the other wave needs
       }
     __syncthreads();
 #pragma unroll
@@ -733,7 +735,7 @@ __global__ __launch_bounds__(256, 2) void gemm_pipe_kernel(elem_t* __restrict__ 
       if ((i < 2) != (wn == 0)) continue;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const f32x4 o = ex[(wm * 64 + j * 16 + r16) * 16 + i * 4 + kg];
+        const f32x4 o = ex[(wm * 64 + j * 16 + r16) * 16 + ((i * 4 + kg) ^ r16)];
         const f32x4 g = wn == 0 ? total[i][j] : o, u = wn == 0 ? o : total[i][j];
         f32x4 y;
         y.x = (g.x * (1.0f / (1.0f + expf(-g.x)))) * u.x;
