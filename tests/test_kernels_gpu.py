@@ -407,7 +407,8 @@ def test_attention_many_decoded_tokens(dtype):
         got = run_attention(k, q_list, kk, vv, P, dtype, window=window, poison=float("nan"), decode_mode=4)
         whole = run_attention(k, q_list, kk, vv, P, dtype, window=window, poison=float("nan"), seed=4, decode_mode=3)
         by_wave = run_attention(k, q_list, kk, vv, P, dtype, window=window, poison=float("nan"), seed=5, decode_mode=5)
-        assert torch.equal(whole, got) and torch.equal(by_wave, got)
+        by_pair = run_attention(k, q_list, kk, vv, P, dtype, window=window, poison=float("nan"), seed=6, decode_mode=7)
+        assert torch.equal(whole, got) and torch.equal(by_wave, got) and torch.equal(by_pair, got)
         for i in (0, 11, 23):
             ref = plain.attention(q_list[i], kk[i], vv[i], d ** -0.5, dtype, window=window)
             torch.testing.assert_close(got[i:i + 1].float(), ref, **tol(dtype))
@@ -420,8 +421,9 @@ def test_attention_many_decoded_tokens(dtype):
                                                (4, 2, 80, 64, 130)])
 def test_attention_decode_kernels_agree(dtype, nq, nkv, d, P, window):
     """Decoded tokens after contexts that end at every place of a tile, a segment and a page, through
-    the kernel with a wave per tile and the one with a wave per segment (head sizes and pages it knows
-    at compile time, and one it does not): the same bits, and the plain result."""
+    the kernel with a wave per tile, the one with a wave per segment and the one with two waves per
+    segment (head sizes and pages they know at compile time, and one they do not): the same bits, and the
+    plain result."""
     k = kern(dtype)
     lens = [1, 2, 63, 64, 65, 255, 256, 257, 320, 511, 512, 513, 1023, 1024, 1025, 1300, 1793, 2047, 2048, 2049]
     q_list = [rand((1, nq, d), dtype, 10 + i) for i in range(len(lens))]
@@ -430,6 +432,9 @@ def test_attention_decode_kernels_agree(dtype, nq, nkv, d, P, window):
     got = run_attention(k, q_list, kk, vv, P, dtype, window=window, poison=float("nan"), decode_mode=4)
     by_wave = run_attention(k, q_list, kk, vv, P, dtype, window=window, poison=float("nan"), seed=5, decode_mode=5)
     assert torch.equal(by_wave, got)
+    # Two waves a segment: segments of one, two, three and four tiles, whole and cut by the context's end or the window.
+    by_pair = run_attention(k, q_list, kk, vv, P, dtype, window=window, poison=float("nan"), seed=6, decode_mode=7)
+    assert torch.equal(by_pair, got)
     for i in range(len(lens)):
         ref = plain.attention(q_list[i], kk[i], vv[i], d ** -0.5, dtype, window=window)
         torch.testing.assert_close(by_wave[i:i + 1].float(), ref, **tol(dtype))

@@ -806,6 +806,136 @@ __global__ __launch_bounds__(64 * SEG_WAVES, 2) void attn_decode_seg_kernel(Attn
   }
 }
 
+// The same with two waves a segment, for steps with so few (token, kv head, segment) triples that a wave each
+// leaves most of the chip idle and every wave waits for its four tiles one after the other: the first wave
+// takes the first half of the segment's tiles, the second wave the rest.  The second wave starts from an empty
+// state, which its first tile fills with that tile's own sums exactly (a fold onto nothing scales by 0 and 1);
+// when the first wave has left its state in LDS, the second folds its own onto it (the fold of that tile onto
+// the tiles before it, as the one wave computes it) and goes on with its other tile: the same bits, and the
+// loads of both halves in flight together.
+template <int DPAD, bool EXACT>
+__global__ __launch_bounds__(128, 2) void attn_decode_pair_kernel(AttnArgs a) {
+  constexpr int NDT = DPAD / 16, NQS = DPAD / VK_SLAB;
+  __shared__ f32x4 hand_acc[NDT][64];
+  __shared__ float hand_ml[2][64];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int G = a.nq / a.nkv, HT = (G + 15) >> 4;
+  const int kvh = blockIdx.y / HT, ht = blockIdx.y - kvh * HT;
+  const int seg = blockIdx.z;
+  const int seq = a.items[2 * blockIdx.x], q_off = a.items[2 * blockIdx.x + 1];
+  const int q_begin = a.cu_q[seq], q_len = a.cu_q[seq + 1] - q_begin;
+  const int k_len = a.k_len[seq];
+  const int tok = q_begin + q_off;
+  const int pos = k_len - q_len + q_off;
+  const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+  const int s0 = max(lo / TILE_KEYS, seg * SEG_TILES), s1 = min(pos / TILE_KEYS, seg * SEG_TILES + SEG_TILES - 1);
+  if (s0 > s1) return;                                  // the whole workgroup
+  const int n = s1 - s0 + 1, n_first = (n + 1) >> 1;
+  const bool paired = n > 1;                            // the same for both waves
+  const int t0 = wave == 0 ? s0 : s0 + n_first, t1 = wave == 0 ? s0 + n_first - 1 : s1;
+  if (t0 > t1) return;                                  // the second wave of a segment with one tile: no barrier follows for the first either
+
+  RowCtx c;
+  init_ctx(c, a, seq, kvh, k_len);
+  c.r16 = lane & 15;
+  c.g = lane >> 4;
+  c.row_ok = c.r16 < min(16, G - ht * 16);
+  c.pos = pos;
+  c.lo = lo;
+  c.wave_lo = lo;
+  const int head = kvh * G + ht * 16 + c.r16;
+  frag_t qf[NQS];
+  load_q<NQS>(a, tok, head, c.row_ok, c.g, qf);
+  frag_t kf[KSUB][NQS];
+  frag_t vf[NDT][KEY_SLABS];
+  load_keys<NQS, EXACT>(c, t0 * TILE_KEYS, kf);
+  load_values<NDT, EXACT>(c, t0 * TILE_KEYS, vf);
+  float M = -INFINITY, L = 0.f;
+  f32x4 ACC[NDT];
+#pragma unroll
+  for (int dt = 0; dt < NDT; ++dt) ACC[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  auto tile = [&](int t, bool more) {
+    const int kb = t * TILE_KEYS;
+    float sc[S_PER_LANE];
+    tile_scores<NQS, EXACT>(c, kf, qf, sc);
+    __builtin_amdgcn_sched_barrier(0);
+    if (more) load_keys<NQS, EXACT>(c, kb + TILE_KEYS, kf);
+    __builtin_amdgcn_sched_barrier(0);
+    const bool full = kb >= lo && kb + TILE_KEYS - 1 <= pos;
+    float m_t, l_t;
+    frag_t pf[KEY_SLABS];
+    tile_softmax(sc, kb, c.g, c.row_ok, lo, pos, c.scale_log2, full, m_t, l_t, pf);
+    const bool seen = m_t > -INFINITY;
+    float Mn, ca, cb;
+    fold_scales(M, m_t, Mn, ca, cb);
+    if (kb + TILE_KEYS > c.k_len || kb < c.wave_lo) {
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt)
+        if (EXACT || dt * 16 < c.d) zero_unowned(vf[dt], kb, c.g, c.wave_lo, c.k_len);
+    }
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) {
+      if (EXACT || dt * 16 < c.d) {
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KEY_SLABS; ++ks) acc = mma_slab(vf[dt][ks], pf[ks], acc);
+        ACC[dt].x = seen ? fold1(ACC[dt].x, acc.x, ca, cb) : ACC[dt].x;
+        ACC[dt].y = seen ? fold1(ACC[dt].y, acc.y, ca, cb) : ACC[dt].y;
+        ACC[dt].z = seen ? fold1(ACC[dt].z, acc.z, ca, cb) : ACC[dt].z;
+        ACC[dt].w = seen ? fold1(ACC[dt].w, acc.w, ca, cb) : ACC[dt].w;
+      }
+    }
+    L = seen ? fold1(L, l_t, ca, cb) : L;
+    M = seen ? Mn : M;
+    __builtin_amdgcn_sched_barrier(0);
+    if (more) load_values<NDT, EXACT>(c, kb + TILE_KEYS, vf);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  // At most two tiles a wave.  The second wave's first tile starts from nothing: its state is then that tile's
+  // own sums; it waits for the first wave's state and folds its own onto it.
+  tile(t0, t0 < t1);
+  if (wave == 1) {
+    __syncthreads();
+    const float Ma = hand_ml[0][lane], La = hand_ml[1][lane];
+    const bool seen = M > -INFINITY;
+    float Mn, ca, cb;
+    fold_scales(Ma, M, Mn, ca, cb);
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) {
+      const f32x4 A = hand_acc[dt][lane];
+      ACC[dt].x = seen ? fold1(A.x, ACC[dt].x, ca, cb) : A.x;
+      ACC[dt].y = seen ? fold1(A.y, ACC[dt].y, ca, cb) : A.y;
+      ACC[dt].z = seen ? fold1(A.z, ACC[dt].z, ca, cb) : A.z;
+      ACC[dt].w = seen ? fold1(A.w, ACC[dt].w, ca, cb) : A.w;
+    }
+    L = seen ? fold1(La, L, ca, cb) : La;
+    M = seen ? Mn : Ma;
+  }
+  if (t0 < t1) tile(t1, false);
+  if (wave == 0 && paired) {
+    // The first half's state, for the second wave (every lane its own part: the same lanes hold the same rows
+    // and columns in both waves).
+    hand_ml[0][lane] = M;
+    hand_ml[1][lane] = L;
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) hand_acc[dt][lane] = ACC[dt];
+    __syncthreads();
+    return;
+  }
+  if (!c.row_ok) return;
+  const int64_t prow = ((int64_t)blockIdx.x * a.nq + head) * a.nseg + seg;
+  if (c.g == 0) {
+    a.part_ml[2 * prow] = M;
+    a.part_ml[2 * prow + 1] = L;
+  }
+  if (M > -INFINITY) {
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt)
+      if (EXACT || dt * 16 < a.d) *reinterpret_cast<f32x4*>(&a.part_acc[prow * a.d + dt * 16 + 4 * c.g]) = ACC[dt];
+  }
+}
+
 // Decoded tokens, all keys of a token in one workgroup: for batches that fill the chip without a
 // split over segments, and contexts whose tile results fit LDS.  Eight waves take the tiles in turn
 // (wave w: tiles first + w, first + w + 8, ...), every tile's (m, l, acc) goes to LDS, and after one
@@ -968,6 +1098,17 @@ int vk_attn_item_rows(void) { return ITEM_ROWS; }
 
 static int vk_dpad(int d) { return d <= 64 ? 64 : (d <= 128 ? 128 : 256); }
 
+static int attn_device_cus() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (cus <= 0) cus = 256;
+  }
+  return cus;
+}
+
 // 1 if prompt rows of this shape go through the kernel that shares key tiles in LDS.
 int vk_attn_prefill_shares_tiles(int d, int P) {
   return (d == 64 || d == 128 || d == 256) && P >= TILE_KEYS && 4 * TILE_KEYS * d * (int)sizeof(elem_t) <= 128 * 1024;
@@ -980,9 +1121,9 @@ int vk_attn_prefill_shares_tiles(int d, int P) {
 //   measurements; the result is the same bits).
 // mode 1: each item is one token; the keys are split by segment over nseg workgroups (nseg must cover
 //   the longest sequence; scratch must hold vk_attn_scratch_floats(n_items, ...)) and folded by a
-//   second kernel; the kernel is chosen by shape.  modes 3, 4, 5: the same through a named kernel
+//   second kernel; the kernel is chosen by shape.  modes 3, 4, 5, 7: the same through a named kernel
 //   (3: all keys of a token in one workgroup where LDS allows, 4: a wave per tile, 5: a wave per
-//   segment; tests and measurements; the same bits).
+//   segment, 7: two waves per segment; tests and measurements; the same bits).
 int vk_paged_attention(elem_t* out, const elem_t* q, const elem_t* kc, const elem_t* vc,
                        const int32_t* block_table, int bt_stride, const int32_t* cu_q, const int32_t* k_len,
                        const int32_t* items, int n_items, int mode, int nseg, float* scratch, int total_tokens,
@@ -992,9 +1133,9 @@ int vk_paged_attention(elem_t* out, const elem_t* q, const elem_t* kc, const ele
   VK_REQUIRE(P >= 8 && (P & (P - 1)) == 0, "attention: page size %d must be a power of two >= 8", P);
   VK_REQUIRE(window >= 0, "attention: window %d must not be negative", window);
   VK_REQUIRE(scale > 0.f, "attention: the score scale must be positive");
-  VK_REQUIRE(mode >= 0 && mode <= 6, "attention: unknown mode %d", mode);
+  VK_REQUIRE(mode >= 0 && mode <= 7, "attention: unknown mode %d", mode);
   const int vk_prefill_variant = mode == 6 ? 14 : 0;
-  const int vk_decode_variant = mode == 3 ? 1 : (mode == 4 ? 2 : (mode == 5 ? 3 : 0));
+  const int vk_decode_variant = mode == 3 ? 1 : (mode == 4 ? 2 : (mode == 5 ? 3 : (mode == 7 ? 4 : 0)));
   if (mode == 6) mode = 0;
   if (mode >= 3) mode = 1;
   if (n_items <= 0) return 0;
@@ -1080,6 +1221,29 @@ int vk_paged_attention(elem_t* out, const elem_t* q, const elem_t* kc, const ele
   // Measured on MI355X, bfloat16, head size 128: from one token of 300 keys (15.5 against 17.2 us)
   // over 8 tokens of 2,060 keys (19 against 25 us) to 64 tokens of 8,231 keys (446 against 506 us)
   // the wave per segment is never slower than the kernel below, nor than the one above.
+  static_assert(SEG_TILES == 4, "the pair kernel gives a wave two tiles at most");
+  // Two waves a segment while there are no more segments in work than one and a quarter per compute unit
+  // (measured on MI355X, head size 128, 8 kv heads, with the fold of the segments; a wave against two waves a
+  // segment: 1 token of 2,090 keys, 72 segments, 14.7 against 12.6 us; 2 tokens, 144: 14.9, 12.9; 4 tokens, 288:
+  // 15.7, 14.9; 8 tokens of 1,000 keys, 256: 14.0, 13.1; 6 tokens of 2,090, 432: 17.5, 19.2; 8 tokens, 576: 19.8,
+  // 21.4; 1 token of 32,800 keys, 1,032: 60.3, 62.0).
+  const bool pair_fits = seg_fits;
+  if (vk_decode_variant == 4 ||
+      (vk_decode_variant == 0 && pair_fits && 4 * (int64_t)grid.x * grid.y * grid.z <= 5 * (int64_t)attn_device_cus())) {
+    const bool exact = P >= TILE_KEYS && d == vk_dpad(d);
+#define DECODE_PAIR(DP)                                                           \
+  do {                                                                            \
+    if (exact) attn_decode_pair_kernel<DP, true><<<grid, 128, 0, st>>>(a);        \
+    else attn_decode_pair_kernel<DP, false><<<grid, 128, 0, st>>>(a);             \
+  } while (0)
+    if (d <= 64) DECODE_PAIR(64);
+    else if (d <= 128) DECODE_PAIR(128);
+    else DECODE_PAIR(256);
+#undef DECODE_PAIR
+    if (vk_check_launch("attention (decoded rows, two waves per segment)")) return 1;
+    attn_combine_kernel<<<dim3(n_items, nq), 64, 0, st>>>(a);
+    return vk_check_launch("attention (combine)");
+  }
   if (vk_decode_variant == 3 || (vk_decode_variant == 0 && seg_fits)) {
     const bool exact = P >= TILE_KEYS && d == vk_dpad(d);
     const dim3 sgrid(grid.x, grid.y, (nseg + SEG_WAVES - 1) / SEG_WAVES);

@@ -349,7 +349,7 @@ void Kernels::paged_attention(Tensor& out, const Tensor& q, const Tensor& k_cach
     throw EngineError("attention: a block table of " + std::to_string(W) + " pages of " + std::to_string(P) + " does not cover " +
                       std::to_string(max_k_len) + " keys");
   void* sp = nullptr;
-  if (mode == 1 || (mode >= 3 && mode <= 5)) {
+  if (mode == 1 || (mode >= 3 && mode <= 5) || mode == 7) {
     if (nseg < (max_k_len + segment_keys_ - 1) / segment_keys_)
       throw EngineError("attention: " + std::to_string(nseg) + " segments do not cover " + std::to_string(max_k_len) + " keys");
     const int64_t need = attn_scratch_floats((int)n_items, (int)nq, (int)d, nseg);

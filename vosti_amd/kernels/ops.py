@@ -326,7 +326,7 @@ class Kernels:
 
         items [n, 2] = (sequence, first row).  mode 0: an item is up to ATTN_ITEM_ROWS consecutive new
         rows of its sequence; modes 2 and 6: the same through a named kernel (same bits); mode 1: an item
-        is a single decoded token; modes 3, 4, 5: the same through a named kernel (same bits; see
+        is a single decoded token; modes 3, 4, 5, 7: the same through a named kernel (same bits; see
         attention.hip).  ``max_k_len`` is the host's bound on k_len; the block table must cover it."""
         T, nq, d = q.shape
         pages, nkv, P, d2 = k_cache.shape
@@ -344,7 +344,7 @@ class Kernels:
         out = torch.empty_like(q) if out is None else out
         self._elem(out, "out", T, nq, d)
         sp = None
-        if mode in (1, 3, 4, 5):
+        if mode in (1, 3, 4, 5, 7):
             need_seg = -(-max_k_len // SEGMENT_KEYS)
             if nseg < need_seg:
                 raise KernelError(f"attention: {nseg} segments do not cover {max_k_len} keys")
