@@ -34,7 +34,8 @@ def rand(shape, dtype, seed, scale=1.0):
                                    (65, 130, 520), (130, 96, 1032), (300, 520, 2056), (8, 40, 4104),
                                    (8, 4100, 1024), (3, 72, 512), (33, 200, 1536), (64, 4096, 4608), (17, 90, 5120),
                                    (40, 6200, 1024), (64, 6144, 512), (23, 24, 2048), (48, 24700, 512), (20, 24576, 1024), (31, 6200, 4096), (17, 100, 1536), (9, 130, 12288), (16, 72, 8704), (2, 40, 5120), (100, 200, 1024), (65, 4100, 512), (130, 96, 1536),
-                                   (250, 8200, 512), (129, 300, 4608), (300, 8400, 128), (700, 9000, 64), (300, 520, 2048), (520, 1000, 4096)])
+                                   (250, 8200, 512), (129, 300, 4608), (300, 8400, 128), (700, 9000, 64), (300, 520, 2048), (520, 1000, 4096),
+                                   (7, 600, 2560), (16, 1000, 3072), (9, 4200, 6144), (3, 264, 5632), (8, 300, 7168), (12, 90, 3584)])
 def test_gemm(dtype, M, N, K):
     k = kern(dtype)
     a, w = rand((M, K), dtype, 1), rand((N, K), dtype, 2, 0.1)
@@ -70,7 +71,8 @@ def test_gemm(dtype, M, N, K):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("N,K", [(4096, 4096), (6144, 1536), (8200, 1024), (24600, 512), (5120, 5120), (300, 8704), (130, 200)])
+@pytest.mark.parametrize("N,K", [(4096, 4096), (6144, 1536), (8200, 1024), (24600, 512), (5120, 5120), (300, 8704), (130, 200),
+                                 (520, 2560), (264, 6144)])
 def test_gemm_every_row_count(dtype, N, K):
     """The kernel is chosen by the sizes, with many borders along the row count (16, 32, 40, 64, 128,
     256, ...): the first M rows of a product are the same bits whatever M is, and so are the fused
@@ -559,11 +561,14 @@ def test_attention_refuses_bad_sizes():
                                    (100, 100, 1024), (300, 256, 2048), (129, 70, 192), (130, 64, 96), (40, 8200, 128),
                                    (8, 100, 5120), (16, 48, 8192), (3, 64, 4608), (32, 4100, 4096), (17, 33, 512),
                                    (64, 200, 1024), (33, 64, 5120), (48, 8200, 512), (20, 130, 4608), (200, 4200, 128), (515, 4500, 64),
-                                   (40, 16384, 512)])
+                                   (40, 16384, 512), (8, 4200, 2560), (2, 100, 3072), (16, 300, 6144), (5, 64, 5632), (11, 72, 7168),
+                                   (9, 40, 2048)])
 def test_gemm_swiglu_fused_equals_separate(dtype, M, I, K):
     """The gate/up projection with the activation folded in (the streaming kernel for few rows, the
     pipelined tile kernel for many, the kernel that shares activations through LDS between them) gives
-    the bits of the two separate kernels; (5, 48, 96), (20, 64, 1024)... with K no multiple of 512 and
+    the bits of the two separate kernels; up to 16 rows the streaming kernel has as many waves a workgroup
+    as K has chunks where that is 2, 4, 5, 6, 10 or 12 (K of 1024, 2048, 2560, 3072, 5120 and 5632, 6144), else
+    eight; (5, 48, 96), (20, 64, 1024)... with K no multiple of 512 and
     (130, 64, 96) fall back to them.  Between 17 and 64 rows a workgroup takes two, three or four gate
     tiles, whichever fills the compute units best: (64, 200, 1024), (48, 8200, 512) and (40, 16384, 512)."""
     k = kern(dtype)

@@ -143,8 +143,8 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_kernel(elem_t* __re
 // a loaded value makes the compiler wait for it at once; and with RC > 0 a wave
 // keeps the activations of its RC chunks (K <= RC * 4096) in registers for the
 // whole kernel.  One barrier per round of eight chunks.
-template <int MT, int W, int RC, int NT>
-__global__ __launch_bounds__(64 * SK_WAVES) void gemm_stream_kernel(elem_t* __restrict__ out,
+template <int MT, int W, int RC, int NT, int NW = SK_WAVES>
+__global__ __launch_bounds__(64 * NW) void gemm_stream_kernel(elem_t* __restrict__ out,
                                                                     const elem_t* __restrict__ act,
                                                                     const elem_t* __restrict__ w, int M, int N, int K,
                                                                     int64_t lda, int64_t ldo, int out_vec_ok) {
@@ -156,8 +156,8 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_stream_kernel(elem_t* __re
   // K <= RC * 8 chunks).  A chunk of one activation tile is 64 registers of 16-bit elements.
   constexpr bool RES = RC > 0;
   static_assert(RC * MT <= 2, "resident activations: at most two chunk tiles per wave");
-  static_assert(NT * MT <= SK_WAVES, "one wave adds up each output tile");
-  __shared__ f32x4 part[2][SK_WAVES][NT * MT][64];
+  static_assert(NT * MT <= NW, "one wave adds up each output tile");
+  __shared__ f32x4 part[2][NW][NT * MT][64];
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r16 = lane & 15, kg = lane >> 4;
@@ -172,7 +172,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_stream_kernel(elem_t* __re
   if (RES) {
 #pragma unroll
     for (int r = 0; r < RC; ++r) {
-      const int c = min(r * SK_WAVES + wave, nchunks - 1);     // beyond K: the last chunk again (not used)
+      const int c = min(r * NW + wave, nchunks - 1);     // beyond K: the last chunk again (not used)
 #pragma unroll
       for (int s = 0; s < KC_SLABS; ++s)
 #pragma unroll
@@ -208,7 +208,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_stream_kernel(elem_t* __re
         for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
       if (c < nchunks) {
         // What this wave streams next: its next chunk of this tile, else its first chunk of the next tile.
-        int nt_ = tile, nc = c + SK_WAVES;
+        int nt_ = tile, nc = c + NW;
         if (nc >= nchunks) {
           nt_ = tile + gridDim.x;
           nc = wave;
@@ -236,7 +236,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_stream_kernel(elem_t* __re
         for (int mt = 0; mt < MT; ++mt) part[parity][wave][nt * MT + mt][lane] = acc[nt][mt];
       __syncthreads();
       if (wave < NT * MT) {
-        for (int w2 = 0; w2 < SK_WAVES; ++w2) {
+        for (int w2 = 0; w2 < NW; ++w2) {
           if (base + w2 < nchunks) {
             const f32x4 p = part[parity][w2][wave][lane];
             total.x = total.x + p.x; total.y = total.y + p.y; total.z = total.z + p.z; total.w = total.w + p.w;
@@ -248,9 +248,9 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_stream_kernel(elem_t* __re
     if (RES) {
 #pragma unroll
       for (int r = 0; r < (RES ? RC : 1); ++r)
-        if (r * SK_WAVES < nchunks) round(r * SK_WAVES, r);
+        if (r * NW < nchunks) round(r * NW, r);
     } else {
-      for (int base = 0; base < nchunks; base += SK_WAVES) round(base, 0);
+      for (int base = 0; base < nchunks; base += NW) round(base, 0);
     }
     if (wave < NT * MT)
       store_out4(out, ldo, (wave % MT) * 16 + r16, (tile * NT + wave / MT) * 16 + 4 * kg, M, N, total, out_vec_ok);
@@ -263,15 +263,15 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_stream_kernel(elem_t* __re
 // two projections rounded to the element type first, which is what the separate
 // GEMM and SwiGLU kernels compute (kernels/triton_kernels/silu_mul.py:64-87).
 // M <= 16, K <= 4096 (activations resident in registers).
-template <int W, int MT, int RC>
-__global__ __launch_bounds__(64 * SK_WAVES) void gemm_stream_swiglu_kernel(elem_t* __restrict__ out,
+template <int W, int MT, int RC, int NW = SK_WAVES>
+__global__ __launch_bounds__(64 * NW) void gemm_stream_swiglu_kernel(elem_t* __restrict__ out,
                                                                            const elem_t* __restrict__ act,
                                                                            const elem_t* __restrict__ w, int M, int I,
                                                                            int K, int64_t lda, int64_t ldo,
                                                                            int out_vec_ok) {
   static_assert(KC_SLABS % W == 0, "the window must divide a chunk");
   static_assert(MT * RC <= 2, "two chunk tiles of activations stay in registers: two tiles of a chunk or two chunks of a tile");
-  __shared__ f32x4 part[2][RC][SK_WAVES][2 * MT][64];      // two sets, used in turn: one barrier per tile
+  __shared__ f32x4 part[2][RC][NW][2 * MT][64];      // two sets, used in turn: one barrier per tile
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r16 = lane & 15, kg = lane >> 4;
@@ -282,7 +282,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_stream_swiglu_kernel(elem_
   frag_t wg[W], wu[W], abuf[RC * KC_SLABS][MT];
 #pragma unroll
   for (int r = 0; r < RC; ++r) {
-    const int c = min(r * SK_WAVES + wave, nchunks - 1);
+    const int c = min(r * NW + wave, nchunks - 1);
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       const elem_t* arow = act + (int64_t)min(mt * 16 + r16, M - 1) * lda + kg * VK_VEC;
@@ -292,11 +292,11 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_stream_swiglu_kernel(elem_
     }
   }
   // Slab g of this wave's stream over a tile: chunk (g / 16) * 8 + wave, slab g % 16 of it.
-  const int my_chunks = wave < nchunks ? (nchunks - wave + SK_WAVES - 1) / SK_WAVES : 0;     // <= RC
+  const int my_chunks = wave < nchunks ? (nchunks - wave + NW - 1) / NW : 0;     // <= RC
   const int my_slabs = my_chunks * KC_SLABS;
   auto issue = [&](int tile, int g, int slot) {
     const int64_t row = min(tile * 16 + r16, I - 1);
-    const int c = (g / KC_SLABS) * SK_WAVES + wave;
+    const int c = (g / KC_SLABS) * NW + wave;
     const elem_t* p = w + row * K + kg * VK_VEC + (int64_t)c * KC + (g % KC_SLABS) * VK_SLAB;
     wg[slot] = *reinterpret_cast<const frag_t*>(p);
     wu[slot] = *reinterpret_cast<const frag_t*>(p + (int64_t)I * K);
@@ -342,8 +342,8 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_stream_swiglu_kernel(elem_
     if (wave < MT) {       // wave mt adds up, in chunk order, and finishes the rows of activation tile mt
       f32x4 tg = {0.f, 0.f, 0.f, 0.f}, tu = {0.f, 0.f, 0.f, 0.f};
       for (int c = 0; c < nchunks; ++c) {
-        const f32x4 pg = part[parity][c / SK_WAVES][c % SK_WAVES][2 * wave][lane];
-        const f32x4 pu = part[parity][c / SK_WAVES][c % SK_WAVES][2 * wave + 1][lane];
+        const f32x4 pg = part[parity][c / NW][c % NW][2 * wave][lane];
+        const f32x4 pu = part[parity][c / NW][c % NW][2 * wave + 1][lane];
         tg.x = tg.x + pg.x; tg.y = tg.y + pg.y; tg.z = tg.z + pg.z; tg.w = tg.w + pg.w;
         tu.x = tu.x + pu.x; tu.y = tu.y + pu.y; tu.z = tu.z + pu.z; tu.w = tu.w + pu.w;
       }
@@ -1146,6 +1146,25 @@ static int device_cus() {
   return cus;
 }
 
+// Waves a workgroup of the streaming kernels at up to 16 rows, for K of nchunks chunks.  Wave w takes the chunks
+// w, w + waves, ...: with eight waves and ten chunks two waves have a second chunk and six wait for them at every
+// tile's barrier, and with two chunks six of eight waves only take up room.  One chunk a wave where a workgroup
+// can be that size (16-bit elements: up to 12 waves; the registers of 32-bit activations allow 8), measured on an
+// MI355X at 8 rows: 34816 gate rows x 5120: 88.6 -> 80.0 us, 7168 x 5120: 23.8 -> 20.4, 2048 x 6144: 12.5 -> 11.2,
+// 151936 x 1024: 103 -> 59, 151936 x 2048: 142 -> 116, 4096 x 1024: 5.5 -> 4.2.  More chunks than that: eight waves
+// (ten or twelve without resident activations: 5120 x 17408 56.8 -> 66 us).
+static int stream_waves(int nchunks) {
+  if (nchunks <= 2) return 2;
+  if (nchunks <= 4) return 4;
+  if (nchunks <= 6) return nchunks;
+  if (nchunks <= 8) return 8;
+#ifdef VK_BF16
+  if (nchunks <= 10) return 10;
+  if (nchunks <= 12) return 12;
+#endif
+  return 8;
+}
+
 // Which kernel computes a product (speed only: all give the same bits).  Every threshold is a count of
 // workgroups against the device's compute units (cus), or a count of 16-row activation tiles, or whether a
 // wave's share of K fits its registers; none is a model's size.  With the workgroups a kernel would start:
@@ -1255,27 +1274,40 @@ int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K
     const int mt = (M + 15) / 16;
     const unsigned grid = (unsigned)((N + 15) / 16);
     if (K % KC == 0) {
-#define ST(MT, W, RC, NT)                                                                                 \
+#define STW(MT, W, RC, NT, NW)                                                                            \
   do {                                                                                                    \
     static int resident = 0; /* workgroups of this kernel that the device holds at once */               \
     if (resident == 0) {                                                                                  \
       int dev = 0, cus = 0, per_cu = 0;                                                                   \
       (void)hipGetDevice(&dev);                                                                           \
       (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);                      \
-      (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gemm_stream_kernel<MT, W, RC, NT>,      \
-                                                         64 * SK_WAVES, 0);                               \
+      (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gemm_stream_kernel<MT, W, RC, NT, NW>,  \
+                                                         64 * NW, 0);                                     \
       resident = (cus > 0 ? cus : 256) * (per_cu > 0 ? per_cu : 1);                                       \
     }                                                                                                     \
     const unsigned groups = (unsigned)((N + 16 * NT - 1) / (16 * NT));                                    \
-    gemm_stream_kernel<MT, W, RC, NT><<<groups < (unsigned)resident ? groups : (unsigned)resident,        \
-                                         64 * SK_WAVES, 0, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok); \
+    gemm_stream_kernel<MT, W, RC, NT, NW><<<groups < (unsigned)resident ? groups : (unsigned)resident,    \
+                                             64 * NW, 0, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok);   \
   } while (0)
+#define ST(MT, W, RC, NT) STW(MT, W, RC, NT, SK_WAVES)
       if (mt == 1) {
         // A few weight tiles more than workgroups in flight (one per compute unit) would mean a second
         // pass of a few: two tiles a workgroup then finish sooner (16 rows, 5120 x 25600: 111 -> 86 us),
         // unless one chunk a wave keeps the activations in registers (6144 x 4096: 12.6 against 15.7 us).
         const int cus = device_cus();
         const int tiles16 = (N + 15) / 16;
+        // One chunk a wave, its activations in registers, wherever a workgroup can have as many waves as K has
+        // chunks (stream_waves): no wave then waits at the round's barrier for one that has a second chunk.
+        const int nw = kernel == 7 ? SK_WAVES : stream_waves(K / KC);
+        if (nw == 2) STW(1, 8, 1, 1, 2);
+        else if (nw == 4) STW(1, 8, 1, 1, 4);
+        else if (nw == 5) STW(1, 8, 1, 1, 5);
+        else if (nw == 6) STW(1, 8, 1, 1, 6);
+#ifdef VK_BF16
+        else if (nw == 10) STW(1, 8, 1, 1, 10);
+        else if (nw == 12) STW(1, 8, 1, 1, 12);
+#endif
+        else
         if (kernel == 7 || (by_size && K > SK_WAVES * KC && tiles16 > cus && 2 * tiles16 <= 3 * cus)) ST(1, 8, 0, 2);
         else if (K <= SK_WAVES * KC) ST(1, 8, 1, 1);
 #ifdef VK_BF16
@@ -1296,6 +1328,7 @@ int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K
       else if (mt == 3) { if (kernel == 7) ST(3, 4, 0, 2); else ST(3, 4, 0, 1); }
       else { if (kernel == 7) ST(4, 4, 0, 2); else ST(4, 4, 0, 1); }
 #undef ST
+#undef STW
       return vk_check_launch("gemm_stream");
     }
 #define SK(MT, W) gemm_skinny_kernel<MT, W><<<grid, 64 * SK_WAVES, 0, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok)
@@ -1372,20 +1405,31 @@ int vk_gemm_swiglu(elem_t* out, const elem_t* act, const elem_t* w, int M, int I
   }
   const int ntiles = (I + 15) / 16;
   const int vec_ok = (ldo % 4 == 0) && ((uintptr_t)out % 16 == 0);
-#define SWIGLU_STREAM(W, MT, RC)                                                                            \
+#define SWIGLU_STREAMW(W, MT, RC, NW)                                                                       \
   do {                                                                                                     \
     static int resident = 0;                                                                               \
     if (resident == 0) {                                                                                   \
       int dev = 0, cus = 0, per_cu = 0;                                                                    \
       (void)hipGetDevice(&dev);                                                                            \
       (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);                       \
-      (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gemm_stream_swiglu_kernel<W, MT, RC>,    \
-                                                         64 * SK_WAVES, 0);                                \
+      (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gemm_stream_swiglu_kernel<W, MT, RC, NW>, \
+                                                         64 * NW, 0);                                      \
       resident = (cus > 0 ? cus : 256) * (per_cu > 0 ? per_cu : 1);                                        \
     }                                                                                                      \
-    gemm_stream_swiglu_kernel<W, MT, RC><<<ntiles < resident ? ntiles : resident, 64 * SK_WAVES, 0, st>>>( \
+    gemm_stream_swiglu_kernel<W, MT, RC, NW><<<ntiles < resident ? ntiles : resident, 64 * NW, 0, st>>>(   \
         out, act, w, M, I, K, lda, ldo, vec_ok);                                                           \
   } while (0)
+#define SWIGLU_STREAM(W, MT, RC) SWIGLU_STREAMW(W, MT, RC, SK_WAVES)
+  const int nw = M <= 16 ? stream_waves(K / KC) : SK_WAVES;       // as in vk_gemm
+  if (nw == 2) SWIGLU_STREAMW(8, 1, 1, 2);
+  else if (nw == 4) SWIGLU_STREAMW(8, 1, 1, 4);
+  else if (nw == 5) SWIGLU_STREAMW(8, 1, 1, 5);
+  else if (nw == 6) SWIGLU_STREAMW(8, 1, 1, 6);
+#ifdef VK_BF16
+  else if (nw == 10) SWIGLU_STREAMW(8, 1, 1, 10);
+  else if (nw == 12) SWIGLU_STREAMW(8, 1, 1, 12);
+#endif
+  else
 #ifdef VK_BF16
   if (M > 16) SWIGLU_STREAM(4, 2, 1);
   else if (K > SK_WAVES * KC) SWIGLU_STREAM(4, 1, 2);
@@ -1393,6 +1437,7 @@ int vk_gemm_swiglu(elem_t* out, const elem_t* act, const elem_t* w, int M, int I
 #endif
     SWIGLU_STREAM(8, 1, 1);
 #undef SWIGLU_STREAM
+#undef SWIGLU_STREAMW
   return vk_check_launch("gemm_swiglu");
 }
 
