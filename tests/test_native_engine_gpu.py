@@ -183,6 +183,34 @@ def test_native_engine_from_python(tiny_dirs, dtype_name, graphs):
         NativeEngine("/nonexistent", dtype=dtype_name)
 
 
+def test_workspace_asked_for_twice_in_one_forward(tmp_path):
+    """A step that is not replayed from a recording, in which the attention asks for the step's workspace twice
+    and for more the second time: 20 decoded rows over 2,310 keys need more floats of partial results than
+    the qkv projection's chunk sums took, and the output projection after them goes through chunk sums again
+    (matrices large enough for that route: 6144 x 2048 and 2048 x 4096).  The buffer of the first request must
+    outlive the second; the tokens are the Python engine's."""
+    import random
+    from vosti_amd.config import Qwen3Config
+    from vosti_amd.engine import NativeEngine
+    from vosti_amd.kernels.ops import SEGMENT_KEYS, kernels_for
+    from vosti_amd.sampling import SamplingParams
+    from vosti_amd.weights import write_random_model
+    cfg = Qwen3Config(vocab_size=1000, hidden_size=2048, intermediate_size=512, num_hidden_layers=1, num_attention_heads=32,
+                      num_key_value_heads=8, head_dim=128, max_position_embeddings=4096, rms_norm_eps=1e-6, rope_theta=1e6,
+                      tie_word_embeddings=False)
+    write_random_model(cfg, 3, tmp_path)
+    k = kernels_for("bfloat16")
+    rows, keys = 20, 2310
+    chunk_sums = k.gemm_workspace_floats(rows, (32 + 2 * 8) * 128, 2048)
+    assert 0 < chunk_sums < k.attn_scratch_floats(rows, 32, 128, -(-keys // SEGMENT_KEYS)) and k.gemm_workspace_floats(rows, 2048, 32 * 128) > 0
+    rng = random.Random(2)
+    ps = [[rng.randrange(1000) for _ in range(keys)] for _ in range(rows)]
+    kw = dict(num_pages=rows * 37 + 8, page_size=64, max_num_seqs=rows, max_num_batched_tokens=8192, graphs=False)
+    sp = SamplingParams(max_tokens=3, ignore_eos=True)
+    want = engine(tmp_path, "bfloat16", **kw).generate(ps, sp)
+    assert NativeEngine(tmp_path, dtype="bfloat16", **kw).generate(ps, sp) == want
+
+
 def test_python_launcher_with_the_native_engine(tiny_dirs, tmp_path):
     """--engine native of the Python launcher prints what --engine python prints (but for the wall time)."""
     import sys

@@ -117,6 +117,7 @@ Tensor ModelRunner::workspace(int64_t floats) {
   }
   Tensor t;
   t.data = workspace_->data();
+  t.owner = workspace_;          // a part may hold this across a later, larger request: the buffer lives as long as the tensor
   t.dtype = DType::F32;
   t.shape = {(int64_t)(workspace_->bytes() / sizeof(float))};
   return t;
@@ -285,6 +286,9 @@ Tensor ModelRunner::run_eager(const std::vector<StepEntry>& entries) {
   std::memcpy(staging_, lay.buf.data(), lay.buf.size() * sizeof(int32_t));
   hip_check(hipMemcpyAsync(meta_->data(), staging_, lay.buf.size() * sizeof(int32_t), hipMemcpyHostToDevice, k_.stream), "step upload");
   hip_check(hipEventRecord(copied_, k_.stream), "event record");
+  // What the parts announced, before the first of them runs: a part that asks twice in its forward (a projection's
+  // chunk sums, then the attention's partial results) then gets the same buffer both times.
+  workspace(workspace_needed(lay.host));
   return forward(lay, static_cast<int32_t*>(meta_->data()));
 }
 

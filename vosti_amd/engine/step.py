@@ -251,6 +251,9 @@ class ModelRunner:
     def _run_eager(self, entries: list[StepEntry]) -> torch.Tensor:
         self.graph_stats["eager"] += 1
         ids, ctx, want = self.build_context(entries)
+        # What the parts announced, before the first of them runs: a part that asks twice in its forward then
+        # gets the same buffer both times.
+        self._get_workspace(self.workspace_needed(ctx.host))
         return self.model.forward(ids, ctx, self.pool.entries, want)
 
     def _run_decode_graph(self, entries: list[StepEntry]) -> torch.Tensor:
