@@ -2,6 +2,7 @@
 """Decode and prefill throughput of the Qwen3-8B shape with random weights on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L]
+    python bench.py --shape 0.6b|1.7b|4b|14b|32b    # the same measurement with the layer sizes of another model of the family
     python bench.py --workload mixed14b     # Qwen3-14B shape: 32 prompts of 128 to 4,096 tokens, prefill in portions beside decoding
     python bench.py --workload prefix32b    # Qwen3-32B shape: 64 requests at context 8,192 that share a 1,024-token prefix
 
@@ -31,6 +32,13 @@ QWEN3_8B = dict(vocab_size=151936, hidden_size=4096, intermediate_size=12288, nu
 # The two larger shapes of the same family, for the other workloads.
 QWEN3_14B = dict(QWEN3_8B, hidden_size=5120, intermediate_size=17408, num_hidden_layers=40, num_attention_heads=40)
 QWEN3_32B = dict(QWEN3_8B, hidden_size=5120, intermediate_size=25600, num_hidden_layers=64, num_attention_heads=64)
+# The family's other sizes, for --shape (the three small ones tie the head to the embedding).
+QWEN3_SHAPES = {
+    "0.6b": dict(QWEN3_8B, hidden_size=1024, intermediate_size=3072, num_hidden_layers=28, num_attention_heads=16, tie_word_embeddings=True),
+    "1.7b": dict(QWEN3_8B, hidden_size=2048, intermediate_size=6144, num_hidden_layers=28, num_attention_heads=16, tie_word_embeddings=True),
+    "4b": dict(QWEN3_8B, hidden_size=2560, intermediate_size=9728, num_hidden_layers=36, tie_word_embeddings=True),
+    "8b": QWEN3_8B, "14b": QWEN3_14B, "32b": QWEN3_32B,
+}
 PROMPT_TOKENS = 2048
 GENERATED_TOKENS = 256
 HBM_PEAK_GBS = 8000.0
@@ -62,7 +70,9 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=None, help="requests (default 8; 64 for prefix32b)")
-    ap.add_argument("--layers", type=int, default=QWEN3_8B["num_hidden_layers"])
+    ap.add_argument("--layers", type=int, default=None, help="layers of the model that is built (default: all of the shape's)")
+    ap.add_argument("--shape", default="8b", choices=sorted(QWEN3_SHAPES), help="which size of the family the decode8b workload takes its "
+                    "layer sizes from (default: the 8B shape, the one the record is about)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--graphs", type=int, default=1, choices=[0, 1], help="replay decode steps from captured HIP graphs")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill timing")
@@ -93,7 +103,11 @@ def main() -> int:
         return other_workload(args)
     if args.batch is None:
         args.batch = 8
-    cfg = Qwen3Config(**dict(QWEN3_8B, num_hidden_layers=args.layers))
+    shape = QWEN3_SHAPES[args.shape]
+    shape_name = f"Qwen3-{args.shape.upper()} shape"
+    if args.layers is None:
+        args.layers = shape["num_hidden_layers"]
+    cfg = Qwen3Config(**dict(shape, num_hidden_layers=args.layers))
     model = build_model(cfg, args.dtype)
     random_weights_on_gpu(model, seed=0)
     torch.cuda.synchronize()
@@ -114,6 +128,7 @@ def main() -> int:
     def decode_run(B: int, steps: int, warmup: int, per_kernel_into: dict | None = None, which: str | None = None):
         """Seconds per decode step of B requests at the context length, and the mean context over the timed steps."""
         which = which or args.engine
+        print(f"bench.py: {shape_name}: {B} requests through the {which} engine", file=sys.stderr, flush=True)
         kw = dict(num_pages=B * pages_per_request, page_size=page, max_num_seqs=B, max_num_batched_tokens=4096,
                   enable_prefix_cache=False, graphs=bool(args.graphs))
         if which == "native":
@@ -167,11 +182,11 @@ def main() -> int:
     bytes_step = decode_bytes(cfg, args.batch, ctx, elem)
     achieved = bytes_step / step_s / 1e9
     record = {
-        "metric": "decode tok/s at batch 8 (+ batch 1/64 and prefill tok/s at 2,048 tok), Qwen3-8B shape",
+        "metric": f"decode tok/s at batch {args.batch} (+ batch 1/64 and prefill tok/s at 2,048 tok), {shape_name}",
         "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dt_name, "data": "synthetic: seeded random token prompts, seeded random weights",
-        "config": {"model": "Qwen3-8B shape", "layers": args.layers, "layers_of_model": QWEN3_8B["num_hidden_layers"],
+        "config": {"model": shape_name, "layers": args.layers, "layers_of_model": shape["num_hidden_layers"],
                    "hidden_size": cfg.hidden_size, "intermediate_size": cfg.intermediate_size,
                    "q_heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
                    "vocab_size": cfg.vocab_size, "global_batch": args.batch, "seq_len": prompt_tokens + GENERATED_TOKENS,
@@ -307,7 +322,7 @@ def other_workload(args) -> int:
 
     shape = QWEN3_14B if args.workload == "mixed14b" else QWEN3_32B
     full_layers = shape["num_hidden_layers"]
-    layers = args.layers if args.layers != QWEN3_8B["num_hidden_layers"] else full_layers
+    layers = args.layers if args.layers is not None else full_layers
     cfg = Qwen3Config(**dict(shape, num_hidden_layers=layers))
     print(f"bench.py: {args.workload}: building {layers} layers", file=sys.stderr, flush=True)
     model = build_model(cfg, args.dtype)
