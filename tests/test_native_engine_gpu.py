@@ -211,6 +211,46 @@ def test_workspace_asked_for_twice_in_one_forward(tmp_path):
     assert NativeEngine(tmp_path, dtype="bfloat16", **kw).generate(ps, sp) == want
 
 
+@pytest.mark.parametrize("dtype_name", ["bfloat16", "float32"])
+def test_busy_workload_at_the_measured_width(tmp_path, dtype_name):
+    """Two layers of the measured model's width, 40 requests: prompts of 20 to 1,500 tokens, half of them behind
+    a shared prefix of 300 tokens, 8 to 70 new tokens each, a third at a temperature, arriving over 30 steps,
+    at most 24 rows and 1,024 tokens a step and a third of the pages they would need together: prompts in
+    portions beside decoding rows, prefix pages found and evicted, requests taken back and computed again,
+    decode steps of 1 to 24 rows replayed from recordings with padding.  Every kernel runs at the sizes of the
+    measurements (17 to 64 rows through chunk sums among them) on memory that the native engine allocates
+    tensor by tensor.  Tokens and statistics are the Python engine's."""
+    import random
+    from vosti_amd.config import Qwen3Config
+    from vosti_amd.engine import NativeEngine
+    from vosti_amd.sampling import SamplingParams
+    from vosti_amd.weights import write_random_model
+    V = 4999
+    cfg = Qwen3Config(vocab_size=V, hidden_size=4096, intermediate_size=12288, num_hidden_layers=2, num_attention_heads=32,
+                      num_key_value_heads=8, head_dim=128, max_position_embeddings=4096, rms_norm_eps=1e-6, rope_theta=1e6,
+                      tie_word_embeddings=False)
+    write_random_model(cfg, 11, tmp_path)
+    rng = random.Random(5)
+    shared = [rng.randrange(V) for _ in range(300)]
+    ps, sp, arrivals = [], [], []
+    for i in range(40):
+        own = [rng.randrange(V) for _ in range(rng.choice((20, 70, 200, 450, 900, 1500)))]
+        ps.append(shared + own if i % 2 else own)
+        sp.append(SamplingParams(max_tokens=rng.randrange(8, 71), temperature=0.7 if i % 3 == 0 else 0.0, seed=i, ignore_eos=True))
+        arrivals.append(rng.randrange(0, 30))
+    need = sum(-(-(len(p) + s.max_tokens) // 64) for p, s in zip(ps, sp))
+    kw = dict(num_pages=need // 3, page_size=64, max_num_seqs=24, max_num_batched_tokens=1024, graphs=True, enable_prefix_cache=True)
+    e = engine(tmp_path, dtype_name, **kw)
+    want = e.generate(ps, sp, arrival_steps=arrivals)
+    assert [len(o) for o in want] == [s.max_tokens for s in sp]
+    native = NativeEngine(tmp_path, dtype=dtype_name, **kw)
+    assert native.generate(ps, sp, arrival_steps=arrivals) == want
+    st = native.stats()
+    assert st["preemptions"] == e.scheduler.preemptions() and st["prefix_hits"] == e.cache.prefix_hits() > 0
+    assert st["graph_stats"] == e.runner.graph_stats and st["graph_stats"]["replayed"] > 20
+    assert st["cache_requests"] == 0 and native.cache_check() == ""
+
+
 def test_python_launcher_with_the_native_engine(tiny_dirs, tmp_path):
     """--engine native of the Python launcher prints what --engine python prints (but for the wall time)."""
     import sys
