@@ -1443,11 +1443,11 @@ int vk_gemm_swiglu(elem_t* out, const elem_t* act, const elem_t* w, int M, int I
 
 
 // float32 elements of workspace that vk_gemm_split needs for these sizes, or 0 if it does not take them:
-// 17 to 64 rows of 16-bit elements, K in whole chunks; rows: weight rows (with swiglu: gate and up rows
+// up to 64 rows of 16-bit elements, K in whole chunks; rows: weight rows (with swiglu: gate and up rows
 // together, an even number of 16-row tiles).
 int64_t vk_gemm_split_floats(int M, int rows, int K, int swiglu) {
 #ifdef VK_BF16
-  if (M <= 16 || M > 64 || rows <= 0 || K <= 0 || K % KC != 0) return 0;
+  if (M <= 0 || M > 64 || rows <= 0 || K <= 0 || K % KC != 0) return 0;
   if (swiglu && rows % 32 != 0) return 0;
   const int mt = (M + 15) / 16;
   return (int64_t)(K / KC) * ((rows + 15) / 16) * mt * 256;
@@ -1457,17 +1457,32 @@ int64_t vk_gemm_split_floats(int M, int rows, int K, int swiglu) {
 #endif
 }
 
-// 1 if the route through chunk sums is the faster one for these sizes (measured with 4096 to 6144 weight rows
-// and K of 4096 and 12288 on an MI355X, 64 rows: 4096 x 12288 45 -> 32 us, 6144 x 4096 20.6 -> 18.2 us, 4096 x
-// 4096 16.0 -> 13.8 us; 32 rows: 41 -> 27, 17.8 -> 14.7, 13.4 -> 11.7 us).  Not with the activation folded in (24576
-// x 4096: 60 -> 62 us), not for matrices of less than 64 KB per compute unit (1000 x 1024 at 32 rows: 4.8 -> 6.5
-// us), and not where workgroups of 128 weight rows are a quarter of the compute units or more: the other
-// kernels then have workgroups enough, and the chunk sums would be a large share of the traffic.
+// 1 if the route through chunk sums is the faster one for these sizes (measured on an MI355X).  Not with the
+// activation folded in (24576 x 4096 at 64 rows: 60 -> 62 us), not for matrices of less than 64 KB per compute
+// unit (1000 x 1024 at 32 rows: 4.8 -> 6.5 us), and not where workgroups of 128 weight rows are a quarter of the
+// compute units or more: the other kernels then have workgroups enough, and the chunk sums would be a large
+// share of the traffic.
+//   17 to 64 rows: always then (64 rows: 4096 x 12288 45 -> 32 us, 6144 x 4096 20.6 -> 18.2, 4096 x 4096 16.0 -> 13.8;
+//     32 rows: 41 -> 27, 17.8 -> 14.7, 13.4 -> 11.7 us).
+//   Up to 16 rows the streaming kernel is the other choice.  With `fill` the share of the compute units that
+//   its last round of one workgroup per 16 weight rows keeps busy:
+//     K of more than 16 chunks (its waves read their activations again for every chunk): when fill < 0.9
+//       (8 rows: 5120 x 17408 56.8 -> 41.7 us, 5120 x 25600 80.8 -> 57.8, 2560 x 9728 19.7 -> 15.3) or from 8 rows on
+//       (4096 x 12288, fill 1: 1 row 23.0 -> 24.5 us, 4 rows 24.7 -> 24.5, 8 rows 27.2 -> 23.9, 16 rows 29.3 -> 24.0);
+//     K of 9 to 16 chunks: when fill < 0.7 (8 rows: 5120 x 5120 18.5 -> 16.6 us, 5120 x 8192 25.9 -> 24.0, 2048 x
+//       6144 11.2 -> 9.6; but 7168 x 5120, fill 0.88, 19.1 -> 21.2);
+//     K of up to 8 chunks: never (4096 x 4096 9.1 -> 10.3 us, 2560 x 4096, fill 0.63, 8.3 -> 9.2).
 int vk_gemm_split_preferred(int M, int rows, int K, int swiglu) {
   if (swiglu || vk_gemm_split_floats(M, rows, K, swiglu) == 0) return 0;
   const int cus = device_cus();
   const int64_t bytes = (int64_t)rows * K * (int64_t)sizeof(elem_t);
-  return bytes >= (int64_t)cus * 65536 && 4 * ((rows + 127) / 128) <= cus;
+  if (bytes < (int64_t)cus * 65536 || 4 * ((rows + 127) / 128) > cus) return 0;
+  if (M > 16) return 1;
+  const int nchunks = K / KC, tiles16 = (rows + 15) / 16;
+  const int rounds = (tiles16 + cus - 1) / cus;
+  const bool fill_below_09 = 10 * tiles16 < 9 * rounds * cus, fill_below_07 = 10 * tiles16 < 7 * rounds * cus;
+  if (nchunks > 2 * SK_WAVES) return fill_below_09 || M >= 8;
+  return nchunks > SK_WAVES && fill_below_07;
 }
 
 // out = act w^T (swiglu 0: w [rows, K], out [M, rows]) or silu(act w_gate^T) * (act w_up^T) (swiglu 1:
@@ -1485,6 +1500,7 @@ int vk_gemm_split(elem_t* out, const elem_t* act, const elem_t* w, int M, int ro
 #ifdef VK_BF16
   const int vec_ok = (ldo % 4 == 0) && ((uintptr_t)out % 16 == 0);
   const int mt = (M + 15) / 16;
+  if (mt == 1) return launch_split<1>(out, act, w, M, rows, K, lda, ldo, swiglu, workspace, vec_ok, st);
   if (mt == 2) return launch_split<2>(out, act, w, M, rows, K, lda, ldo, swiglu, workspace, vec_ok, st);
   if (mt == 3) return launch_split<3>(out, act, w, M, rows, K, lda, ldo, swiglu, workspace, vec_ok, st);
   return launch_split<4>(out, act, w, M, rows, K, lda, ldo, swiglu, workspace, vec_ok, st);
