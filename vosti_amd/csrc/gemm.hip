@@ -13,13 +13,17 @@
 // kernels/triton_kernels/qkv_matmul.py:24-32).
 //
 //   gemm_stream         M <= 64, K a multiple of 512.  Streams the weights once from HBM: persistent
-//                       workgroups of eight waves walk over 16-row weight tiles (one or two at a time);
-//                       wave w takes the chunks w, w+8, ... and keeps a rolling window of slabs in
-//                       flight, also across tile borders.  After each round of eight chunks the chunk
-//                       sums meet in LDS and are added in chunk order.
+//                       workgroups walk over 16-row weight tiles (one or two at a time); wave w of a
+//                       workgroup's W waves takes the chunks w, w+W, ... and keeps a rolling window of
+//                       slabs in flight, also across tile borders.  After each round of W chunks the chunk
+//                       sums meet in LDS and are added in chunk order.  W is eight, or, up to 16 rows, the
+//                       number of chunks where that is 2, 4, 5, 6, 10 or 12 (stream_waves).
 //   gemm_stream_swiglu  the same for the gate/up projection with SwiGLU folded in (M <= 16).
 //   gemm_mid            17 <= M <= 64, K a multiple of 512: 64 or 32 weight rows per workgroup, weights
 //                       streamed into registers, the activations of the chunks in work shared through LDS.
+//   gemm_split          M <= 64, K a multiple of 512, 16-bit elements, with a workspace: a workgroup per
+//                       (128 weight rows, chunk) leaves its chunk sums in the workspace, a second kernel
+//                       adds them in chunk order (vk_gemm_split; vk_gemm_split_preferred says when).
 //   gemm_skinny         M <= 64, any K: the same decomposition with predicated loads.
 //   gemm_pipe           any M, K a multiple of two slabs (128 bytes of a row): 128x128 output tile per
 //                       workgroup, 64x64 per wave, tiles straight from global memory into LDS, two
@@ -1197,7 +1201,7 @@ static int stream_waves(int nchunks) {
 //              two blocks                                      9 (wg32 <= 0.5 cus) or 8
 //              else                                            2 (k_resident and wg16 >= 1.5 cus) or 8
 //   more                                                       2   the pipelined tile kernel
-// With a workspace the products of 17 to 64 rows that vk_gemm_split_preferred names go through chunk sums
+// With a workspace the products of up to 64 rows that vk_gemm_split_preferred names go through chunk sums
 // instead (the caller's choice: vk_gemm_split).
 static int choose_gemm_kernel(int M, int N, int K) {
   const int cus = device_cus();
