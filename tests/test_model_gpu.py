@@ -227,11 +227,21 @@ def test_trace_run_program(tiny_dirs, plain_logits, tmp_path, dtype_name):
         {"step": 4, "entries": [{"id": "c", "tokens": prompts[c], "want": [119]}], "end": ["c"]},
     ]
     run_trace(tiny_dirs[name], dtype_name, tmp_path, max_tokens=128 + 192, steps=steps)
-    read = lambda s: torch.from_numpy(np.fromfile(tmp_path / f"{s}.f32", dtype="<f4").reshape(-1, vocab))
+    read = lambda s, d=tmp_path: torch.from_numpy(np.fromfile(d / f"{s}.f32", dtype="<f4").reshape(-1, vocab))
     # The few rows that were asked for, against the same rows of the plain logits.
     got = torch.cat([read(s) for s in range(5)])
     pick = lambda t: torch.cat([t[a][[0, 39]], t[a][[64]], t[b][[127]], t[b][[128]], t[c][[119]]])
     assert_matches_plain(got, pick(ref), pick(exact), dtype_name, "trace_run")
+    # The same trace through the native engine's step function: the same kernels and cache manager under other
+    # host code, so the same bits (the frequencies of the rotation come from another pow routine, which may
+    # differ in the last bit of an entry: then the logits do, and the comparison with the plain ones decides).
+    native_dir = tmp_path / "native"
+    native_dir.mkdir()
+    run_trace(tiny_dirs[name], dtype_name, native_dir, max_tokens=128 + 192, steps=steps, extra=["--engine", "native"])
+    got_native = torch.cat([read(s, native_dir) for s in range(5)])
+    if not torch.equal(got_native, got):
+        assert_matches_plain(got_native, pick(ref), pick(exact), dtype_name, "trace_run --engine native")
+        assert (got_native - got).abs().max() <= (got - pick(exact)).abs().max()
 
 
 FULL_WIDTH = dict(vocab_size=4999, hidden_size=4096, intermediate_size=12288, num_hidden_layers=2, num_attention_heads=32,
@@ -408,19 +418,20 @@ def test_trace_run_prefix_reuse_is_bit_identical_to_a_cold_run(tiny_dirs, tmp_pa
         steps = [{"step": 0, "entries": [{"id": "a", "prompt": a, "tokens": a, "want": [len(a) - 1]}], "end": ["a"]},
                  {"step": 1, "entries": [{"id": "b", "prompt": b, "tokens": b[:80], "want": [w for w in want_b if w < 80]}], "end": []},
                  {"step": 2, "entries": [{"id": "b", "tokens": b[80:], "want": [w - 80 for w in want_b if w >= 80]}], "end": ["b"]}]
-        extra = ["--prefix-cache", "--prefix-report", str(out / "report.txt")] if warm else []
+        extra = (["--prefix-cache", "--prefix-report", str(out / "report.txt")] if warm else []) + ["--engine", which]
         run_trace(tiny_dirs[name], dtype_name, out, max_tokens=256, steps=steps, page_size=page, extra=extra)
         return [np.fromfile(out / f"{s}.f32", dtype="<f4").reshape(-1, vocab) for s in range(3)]
 
-    cold_dir, warm_dir = tmp_path / "cold", tmp_path / "warm"
-    cold_dir.mkdir(); warm_dir.mkdir()
-    cold, warm = run(cold_dir, False), run(warm_dir, True)
-    report = dict(line.split() for line in (warm_dir / "report.txt").read_text().splitlines())
-    cached = 70 // page * page
-    assert report == {"a": "0", "b": str(cached)} and cached > 0          # b found a's pages
-    assert np.array_equal(warm[0], cold[0])
-    assert warm[1].shape[0] == 80 - cached and np.array_equal(warm[1], cold[1][cached:])    # the cached tokens are not run
-    assert np.array_equal(warm[2], cold[2])
+    for which in ("python", "native"):        # the two step functions, each cold against warm
+        cold_dir, warm_dir = tmp_path / f"cold_{which}", tmp_path / f"warm_{which}"
+        cold_dir.mkdir(); warm_dir.mkdir()
+        cold, warm = run(cold_dir, False), run(warm_dir, True)
+        report = dict(line.split() for line in (warm_dir / "report.txt").read_text().splitlines())
+        cached = 70 // page * page
+        assert report == {"a": "0", "b": str(cached)} and cached > 0          # b found a's pages
+        assert np.array_equal(warm[0], cold[0])
+        assert warm[1].shape[0] == 80 - cached and np.array_equal(warm[1], cold[1][cached:])    # the cached tokens are not run
+        assert np.array_equal(warm[2], cold[2])
 
 
 @pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])

@@ -251,6 +251,66 @@ def test_busy_workload_at_the_measured_width(tmp_path, dtype_name):
     assert st["cache_requests"] == 0 and native.cache_check() == ""
 
 
+class _NativeRunner:
+    """The native engine's step function behind the face that test_model_gpu's replay() drives."""
+
+    class _Cache:
+        def __init__(self, engine):
+            self.engine = engine
+
+        def num_requests(self):
+            return self.engine.stats()["cache_requests"]
+
+        def check(self):
+            return self.engine.cache_check()
+
+    class _Identity:
+        @staticmethod
+        def to_f32(x):
+            return x
+
+    def __init__(self, model_dir, dtype_name, page_size, num_pages):
+        from vosti_amd.engine import NativeEngine
+        self.engine = NativeEngine(model_dir, dtype=dtype_name, num_pages=num_pages, page_size=page_size, max_num_seqs=8,
+                                   enable_prefix_cache=False, graphs=False)
+        self.cache, self.kernels = self._Cache(self.engine), self._Identity()
+
+    def step(self, entries):
+        return torch.from_numpy(self.engine.trace_step([(e.request_id, e.tokens, e.want) for e in entries]))
+
+    def finish(self, rid):
+        self.engine.trace_finish(rid)
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_every_cutting_through_the_native_step_function(tiny_dirs, name, dtype_name):
+    """The native engine's step function under the four cuttings of the Python one's test: every request alone
+    and whole; all but the last 32 tokens in one step and the rest one by one; portions of changing size down to
+    one token; up to four live requests mixed, on so few pages that they are used again.  The logits of every
+    (request, position) are the same bits under all four, and the whole prompts' are the Python step function's
+    (where a rotation frequency differs in its last bit between the two pow routines, within that bit's reach)."""
+    from test_model_gpu import cut_chunks, cut_mixed, cut_tail, cut_whole, make_runner, prompts_for, replay, LENGTHS
+    prompts = prompts_for(name)
+    page = TINY[name][1]
+    mixed_steps, mixed_pages = cut_mixed(prompts, page)
+    pages = -(-max(LENGTHS[name]) // page)
+    runner = _NativeRunner(tiny_dirs[name], dtype_name, page, pages)
+    whole = replay(runner, cut_whole(prompts))
+    for label, steps, n in (("tail", cut_tail(prompts), None), ("chunks", cut_chunks(prompts), None), ("mixed", mixed_steps, mixed_pages)):
+        if n is not None:
+            runner = _NativeRunner(tiny_dirs[name], dtype_name, page, n)
+        got = replay(runner, steps)
+        assert set(got) == set(whole), label
+        bad = [k for k in sorted(whole) if not torch.equal(got[k], whole[k])]
+        assert not bad, f"{label}: first differing (request, position) {bad[:1]} of {len(bad)}"
+    py = replay(make_runner(tiny_dirs[name], dtype_name, page, num_pages=pages), cut_whole(prompts))
+    differing = [k for k in sorted(whole) if not torch.equal(py[k], whole[k])]
+    if differing:
+        worst = max((py[k] - whole[k]).abs().max().item() for k in differing)
+        assert worst < (2e-2 if dtype_name == "bfloat16" else 1e-4), (len(differing), worst)
+
+
 def test_python_launcher_with_the_native_engine(tiny_dirs, tmp_path):
     """--engine native of the Python launcher prints what --engine python prints (but for the wall time)."""
     import sys

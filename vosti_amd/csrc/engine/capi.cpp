@@ -17,7 +17,7 @@ void put(char* err, int cap, const std::string& text) {
 
 extern "C" {
 
-int ve_abi_version(void) { return 1; }
+int ve_abi_version(void) { return 2; }
 
 // dtype: "bf16" or "f32".  random_weights != 0: the folder needs config.json only and the weights are drawn
 // from `seed` on the GPU.
@@ -105,6 +105,65 @@ void ve_stats(void* h, int64_t* out) {
   out[7] = e->cache().num_requests();
   out[8] = e->model().spec().vocab_size;
   out[9] = e->model().spec().max_positions;
+}
+
+// ---- The step function alone, for replaying given tokens (no scheduler, no sampling).  An engine is used either
+// this way or through ve_add_request / ve_step, not both: the two share the cache manager.
+
+// Announces a request's whole prompt so that cached pages can be matched (with the prefix cache on).  Returns the
+// number of its first tokens that are cached already, or -1.
+int ve_trace_add_request(void* h, int64_t id, const int32_t* prompt, int n_prompt, char* err, int errcap) {
+  try {
+    int cached = 0;
+    const Status st = static_cast<Engine*>(h)->cache().add_request((RequestId)id, prompt, n_prompt, &cached);
+    if (st != OK) throw EngineError("request " + std::to_string(id) + " was refused by the cache manager (status " + std::to_string((int)st) + ")");
+    return cached;
+  } catch (const std::exception& e) {
+    put(err, errcap, e.what());
+    return -1;
+  }
+}
+
+// One step: entry i is request ids[i] with the next tokens[tok_off[i] .. tok_off[i + 1]) and the wanted places
+// want[want_off[i] .. want_off[i + 1]) among them.  The logits at the wanted places, in the order of the entries and
+// of `want`, go to `out` as float32 [wanted, vocabulary] (room for out_floats).  Returns the wanted rows, or -1.
+int64_t ve_trace_step(void* h, int n_entries, const int64_t* ids, const int32_t* tok_off, const int32_t* tokens,
+                      const int32_t* want_off, const int32_t* want, float* out, int64_t out_floats, char* err, int errcap) {
+  try {
+    Engine* e = static_cast<Engine*>(h);
+    std::vector<StepEntry> entries((size_t)(n_entries > 0 ? n_entries : 0));
+    for (int i = 0; i < n_entries; ++i) {
+      entries[i].id = (RequestId)ids[i];
+      entries[i].tokens.assign(tokens + tok_off[i], tokens + tok_off[i + 1]);
+      entries[i].want.assign(want + want_off[i], want + want_off[i + 1]);
+    }
+    const Tensor logits = e->runner().step(entries);
+    const int64_t rows = logits.numel() ? logits.dim(0) : 0;
+    if (rows > 0) {
+      if (logits.numel() > out_floats) throw EngineError("the caller's buffer is too small for the wanted logits");
+      Kernels& k = e->model().kernels();
+      const Tensor f = k.to_f32(logits);
+      hip_check(hipMemcpyAsync(out, f.data, f.bytes(), hipMemcpyDeviceToHost, k.stream), "logits readback");
+    }
+    e->synchronize();
+    return rows;
+  } catch (const std::exception& e) {
+    put(err, errcap, e.what());
+    return -1;
+  }
+}
+
+int ve_trace_has_request(void* h, int64_t id) { return static_cast<Engine*>(h)->cache().has_request((RequestId)id) ? 1 : 0; }
+
+// The request is over: what it holds is given back.
+int ve_trace_finish(void* h, int64_t id, char* err, int errcap) {
+  try {
+    static_cast<Engine*>(h)->runner().finish((RequestId)id);
+    return 0;
+  } catch (const std::exception& e) {
+    put(err, errcap, e.what());
+    return -1;
+  }
 }
 
 // Writes the cache manager's first violated invariant into buf (empty if none); returns its length.

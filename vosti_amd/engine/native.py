@@ -20,7 +20,7 @@ from ..kernels import build
 from ..kernels.ops import dtype_name
 from ..sampling import SamplingParams
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 _LIB = None
 
 
@@ -48,6 +48,11 @@ def _lib():
         lib.ve_synchronize.argtypes = [c_void_p, c_char_p, c_int]
         lib.ve_stats.argtypes = [c_void_p, c_void_p]
         lib.ve_cache_check.argtypes = [c_void_p, c_char_p, c_int]
+        lib.ve_trace_add_request.argtypes = [c_void_p, c_int64, c_void_p, c_int, c_char_p, c_int]
+        lib.ve_trace_step.restype = c_int64
+        lib.ve_trace_step.argtypes = [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_char_p, c_int]
+        lib.ve_trace_has_request.argtypes = [c_void_p, c_int64]
+        lib.ve_trace_finish.argtypes = [c_void_p, c_int64, c_char_p, c_int]
         _LIB = lib
     return _LIB
 
@@ -120,6 +125,39 @@ class NativeEngine:
         buf = ctypes.create_string_buffer(1024)
         self._lib.ve_cache_check(self._h, buf, len(buf))
         return buf.value.decode()
+
+    # --------------------------------------------------------------- replay
+    # The step function alone (what bin/trace_run drives): given tokens in, logits out; no scheduler, no sampling.
+    # An engine is used either this way or through add_request / step, not both.
+    def trace_add_request(self, rid: int, prompt: list[int]) -> int:
+        """Announces a request's whole prompt (prefix cache on); returns how many of its first tokens are cached."""
+        p = np.asarray(prompt, dtype=np.int32)
+        cached = self._lib.ve_trace_add_request(self._h, rid, p.ctypes.data, len(p), self._err, len(self._err))
+        if cached < 0:
+            self._fail()
+        return cached
+
+    def trace_step(self, entries: list[tuple[int, list[int], list[int]]]) -> np.ndarray:
+        """entries: (request id, its next tokens, wanted places among them).  float32 logits [wanted, vocabulary]."""
+        ids = np.asarray([e[0] for e in entries], dtype=np.int64)
+        tok_off = np.cumsum([0] + [len(e[1]) for e in entries], dtype=np.int64).astype(np.int32)
+        want_off = np.cumsum([0] + [len(e[2]) for e in entries], dtype=np.int64).astype(np.int32)
+        tokens = np.asarray([t for e in entries for t in e[1]], dtype=np.int32)
+        want = np.asarray([w for e in entries for w in e[2]], dtype=np.int32)
+        vocab = self.stats()["vocab_size"]
+        out = np.empty((int(want_off[-1]), vocab), dtype=np.float32)
+        rows = self._lib.ve_trace_step(self._h, len(entries), ids.ctypes.data, tok_off.ctypes.data, tokens.ctypes.data,
+                                       want_off.ctypes.data, want.ctypes.data, out.ctypes.data, out.size, self._err, len(self._err))
+        if rows < 0:
+            self._fail()
+        return out[:rows]
+
+    def trace_has_request(self, rid: int) -> bool:
+        return bool(self._lib.ve_trace_has_request(self._h, rid))
+
+    def trace_finish(self, rid: int) -> None:
+        if self._lib.ve_trace_finish(self._h, rid, self._err, len(self._err)) != 0:
+            self._fail()
 
     # ------------------------------------------------------------- generate
     def generate(self, prompts: list[list[int]], params: SamplingParams | list[SamplingParams] | None = None,

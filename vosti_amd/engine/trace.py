@@ -20,6 +20,9 @@ def build_parser() -> argparse.ArgumentParser:
     p.add_argument("--prefix-cache", action="store_true",
                    help="a request whose first tokens equal full pages that an earlier request left reuses those pages: "
                         "feed such a request its tokens from the first uncached one on (--prefix-report tells which)")
+    p.add_argument("--engine", default="python", choices=["python", "native"],
+                   help="which step function runs the trace: the Python one (engine/step.py) or the native engine's "
+                        "(csrc/engine/runner.cpp); the same kernels, cache manager and logits")
     p.add_argument("--prefix-report", default=None,
                    help="a file that gets one line '<id> <cached tokens>' when a request with a 'prompt' field is first seen")
     return p
@@ -34,16 +37,33 @@ def main(argv: list[str] | None = None) -> int:
     if not torch.cuda.is_available():
         print("trace_run: no GPU visible; this engine has no CPU path", file=sys.stderr)
         return 2
-    from ..cache import CachePool
-    from ..models import load_model
-    from .step import ModelRunner, StepEntry
-
-    model = load_model(args.model, args.dtype)
     page = args.page_size
     num_pages = max(1, -(-args.max_tokens // page))
-    pool = CachePool(model, page_size=page, num_pages=num_pages, num_slots=args.max_requests,
-                     prefix_cache=args.prefix_cache)
-    runner = ModelRunner(model, pool)
+    if args.engine == "native":
+        from .native import NativeEngine
+        native = NativeEngine(args.model, dtype=args.dtype, num_pages=num_pages, page_size=page, max_num_seqs=args.max_requests,
+                              enable_prefix_cache=args.prefix_cache, graphs=False)
+        add_request, has_request, finish = native.trace_add_request, native.trace_has_request, native.trace_finish
+
+        def step_logits(entries):
+            return native.trace_step(entries)
+    else:
+        from ..cache import CachePool
+        from ..models import load_model
+        from .step import ModelRunner, StepEntry
+
+        model = load_model(args.model, args.dtype)
+        pool = CachePool(model, page_size=page, num_pages=num_pages, num_slots=args.max_requests,
+                         prefix_cache=args.prefix_cache)
+        runner = ModelRunner(model, pool)
+        add_request, has_request, finish = runner.cache.add_request, runner.cache.has_request, runner.finish
+
+        def step_logits(entries):
+            logits = runner.step([StepEntry(*e) for e in entries])
+            if logits.shape[0] == 0:
+                torch.cuda.synchronize()
+                return np.empty((0, 0), dtype=np.float32)
+            return model.kernels.to_f32(logits).cpu().numpy()
     report = open(args.prefix_report, "a") if args.prefix_report else None
     out_dir = Path(args.out)
     out_dir.mkdir(parents=True, exist_ok=True)
@@ -65,7 +85,7 @@ def main(argv: list[str] | None = None) -> int:
                 if args.prefix_cache and "prompt" in e:
                     # The whole prompt is announced so that cached pages can be matched; the entry's tokens
                     # must then start right after the cached ones, which are not computed again.
-                    cached = runner.cache.add_request(ids[name], [int(t) for t in e["prompt"]])
+                    cached = add_request(ids[name], [int(t) for t in e["prompt"]])
                     if report:
                         report.write(f"{name} {cached}\n")
                         report.flush()
@@ -73,18 +93,15 @@ def main(argv: list[str] | None = None) -> int:
                     if skip < 0:
                         raise SystemExit(f"trace_run: request {name} starts at {e.get('start', 0)} but {cached} tokens are cached")
                     e = dict(e, tokens=e["tokens"][skip:], want=[w - skip for w in e.get("want", []) if w >= skip])
-            entries.append(StepEntry(ids[name], [int(t) for t in e["tokens"]], [int(w) for w in e.get("want", [])]))
-        logits = runner.step(entries)
+            entries.append((ids[name], [int(t) for t in e["tokens"]], [int(w) for w in e.get("want", [])]))
+        logits = step_logits(entries)
         if logits.shape[0] > 0:
-            arr = model.kernels.to_f32(logits).cpu().numpy().astype("<f4", copy=False)
-            arr.tofile(str(out_dir / f"{step}.f32"))
-        else:
-            torch.cuda.synchronize()
+            logits.astype("<f4", copy=False).tofile(str(out_dir / f"{step}.f32"))
         for name in rec.get("end", []):
             name = str(name)
             if name in ids:
                 rid = ids.pop(name)
-                if runner.cache.has_request(rid):
-                    runner.finish(rid)
+                if has_request(rid):
+                    finish(rid)
         print(f"done {step}", flush=True)
     return 0
