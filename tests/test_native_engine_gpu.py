@@ -311,6 +311,43 @@ def test_every_cutting_through_the_native_step_function(tiny_dirs, name, dtype_n
         assert worst < (2e-2 if dtype_name == "bfloat16" else 1e-4), (len(differing), worst)
 
 
+FAMILY_WIDTHS = {       # hidden, inside, q heads, kv heads (head size 128): the layer sizes of the family's models
+    "0.6b": (1024, 3072, 16, 8), "1.7b": (2048, 6144, 16, 8), "4b": (2560, 9728, 32, 8), "14b": (5120, 17408, 40, 8), "32b": (5120, 25600, 64, 8),
+}
+
+
+@pytest.mark.parametrize("shape", sorted(FAMILY_WIDTHS))
+def test_the_family_s_other_widths_through_both_engines(tmp_path, shape):
+    """One layer of each of the family's other layer sizes (the projections then take other kernels: two to twelve
+    waves a workgroup in the streaming kernels, the route through chunk sums at other row counts, other tile
+    grids) under a small staggered workload with recorded decode steps of 1 to 20 rows and prompts in portions:
+    the native engine's tokens are the Python engine's, and the first request's are the plain implementation's
+    choices within the type's cost."""
+    import random
+    from vosti_amd.config import Qwen3Config
+    from vosti_amd.engine import NativeEngine
+    from vosti_amd.sampling import SamplingParams
+    from vosti_amd.weights import write_random_model
+    H, I, nq, nkv = FAMILY_WIDTHS[shape]
+    V = 2003
+    cfg = Qwen3Config(vocab_size=V, hidden_size=H, intermediate_size=I, num_hidden_layers=1, num_attention_heads=nq,
+                      num_key_value_heads=nkv, head_dim=128, max_position_embeddings=2048, rms_norm_eps=1e-6, rope_theta=1e6,
+                      tie_word_embeddings=H <= 2560)
+    write_random_model(cfg, 21, tmp_path)
+    rng = random.Random(len(shape) + H)
+    ps = [[rng.randrange(V) for _ in range(rng.choice((5, 40, 130, 300, 700)))] for _ in range(20)]
+    sp = [SamplingParams(max_tokens=rng.randrange(6, 30), temperature=0.6 if i % 4 == 1 else 0.0, seed=i, ignore_eos=True) for i in range(20)]
+    arrivals = [rng.randrange(0, 12) for _ in ps]
+    kw = dict(num_pages=20 * 12, page_size=64, max_num_seqs=20, max_num_batched_tokens=512, graphs=True)
+    e = engine(tmp_path, "bfloat16", **kw)
+    want = e.generate(ps, sp, arrival_steps=arrivals)
+    native = NativeEngine(tmp_path, dtype="bfloat16", **kw)
+    assert native.generate(ps, sp, arrival_steps=arrivals) == want
+    assert native.stats()["graph_stats"] == e.runner.graph_stats and native.cache_check() == ""
+    first = next(i for i in range(20) if sp[i].temperature == 0.0 and len(ps[i]) <= 130)
+    check_greedy_against_plain(PlainQwen3(tmp_path, torch.bfloat16), ps[first], want[first], "bfloat16", PlainQwen3(tmp_path, torch.float32))
+
+
 def test_python_launcher_with_the_native_engine(tiny_dirs, tmp_path):
     """--engine native of the Python launcher prints what --engine python prints (but for the wall time)."""
     import sys
