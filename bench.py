@@ -257,14 +257,18 @@ def kernel_times(model, cfg, pool, M: int, keys: int, elem: int, decode: bool) -
                                                 max_k_len=M, out=out)
     layers = model.layers
     o_qkv, o_h, o_i, o_attn = k.empty(M, (nq + 2 * nkv) * d), k.empty(M, H), k.empty(M, I), k.empty(M, nq, d)
+    # The step's workspace, as the parts ask for it: with it some projections take the route through chunk sums.
+    need = max(k.gemm_workspace_floats(M, rows_, K_, swiglu=sw) for rows_, K_, sw in
+               (((nq + 2 * nkv) * d, H, False), (H, nq * d, False), (2 * I, H, True), (H, I, False)))
+    ws = torch.empty(max(need, 1), dtype=torch.float32, device="cuda")
     head_rows = M if decode else 1
     o_v = k.empty(head_rows, V)
     work = {
-        "qkv": (lambda l: k.gemm(x, layers[l].mixer.w_qkv, out=o_qkv), (nq + 2 * nkv) * d * H, L),
+        "qkv": (lambda l: k.gemm(x, layers[l].mixer.w_qkv, out=o_qkv, workspace=ws), (nq + 2 * nkv) * d * H, L),
         "attention": (lambda l: attn(pool.entries[l], o_attn), None, L),
-        "o": (lambda l: k.gemm(a, layers[l].mixer.w_o, out=o_h), H * nq * d, L),
-        "gate_up": (lambda l: k.gemm_swiglu(x, layers[l].feed_forward.w_gate_up), 2 * I * H, L),
-        "down": (lambda l: k.gemm(m, layers[l].feed_forward.w_down, out=o_h), H * I, L),
+        "o": (lambda l: k.gemm(a, layers[l].mixer.w_o, out=o_h, workspace=ws), H * nq * d, L),
+        "gate_up": (lambda l: k.gemm_swiglu(x, layers[l].feed_forward.w_gate_up, workspace=ws), 2 * I * H, L),
+        "down": (lambda l: k.gemm(m, layers[l].feed_forward.w_down, out=o_h, workspace=ws), H * I, L),
         "lm_head": (lambda l: k.gemm(x[:head_rows], model.head.weight, out=o_v), V * H, 1),
     }
     out = {}
