@@ -273,7 +273,8 @@ def kernel_times(model, cfg, pool, M: int, keys: int, elem: int, decode: bool) -
     }
     out = {}
     reps = 5
-    for name, (fn, weight_elems, calls) in work.items():
+
+    def time_calls(fn, calls):
         for l in range(calls):                      # warm: every kernel variant is loaded before the capture
             fn(l)
         torch.cuda.synchronize()
@@ -289,7 +290,16 @@ def kernel_times(model, cfg, pool, M: int, keys: int, elem: int, decode: bool) -
             graph.replay()
         t1.record()
         torch.cuda.synchronize()
-        us = t0.elapsed_time(t1) * 1e3 / (reps * calls)
+        return t0.elapsed_time(t1) * 1e3 / (reps * calls)
+
+    # The yardstick for the decode projections: a kernel that only reads the same weights, launch after launch
+    # like them (what such reads reach on this machine, well below the 8 TB/s that the fractions are priced at).
+    sink = torch.zeros(1, dtype=torch.int32, device="cuda")
+    weights = {"qkv": lambda l: layers[l].mixer.w_qkv, "o": lambda l: layers[l].mixer.w_o,
+               "gate_up": lambda l: layers[l].feed_forward.w_gate_up, "down": lambda l: layers[l].feed_forward.w_down,
+               "lm_head": lambda l: model.head.weight}
+    for name, (fn, weight_elems, calls) in work.items():
+        us = time_calls(fn, calls)
         rows = head_rows if name == "lm_head" else M
         if name == "attention":
             flops = 4.0 * nq * d * (M * keys if decode else M * (M + 1) / 2)
@@ -299,10 +309,12 @@ def kernel_times(model, cfg, pool, M: int, keys: int, elem: int, decode: bool) -
         if decode or name == "lm_head":      # one row through the head is a read of its weights, whatever the step
             gbps = nbytes / us / 1e3
             out[name] = {"us": round(us, 2), "GBps": round(gbps, 1), "frac": round(gbps / HBM_PEAK_GBS, 3)}
+            if name in weights:
+                pull_us = time_calls(lambda l, get=weights[name]: k.pull(get(l), sink), calls)
+                out[name].update(read_only_us=round(pull_us, 2), frac_of_read_only=round(pull_us / us, 3))
         else:
             tf = flops / us / 1e6
             out[name] = {"us": round(us, 2), "TFLOPs": round(tf, 1), "frac": round(tf * 1e12 / PEAK_FLOPS[dt_name], 3)}
-        del graph
     return out
 
 

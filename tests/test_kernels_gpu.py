@@ -583,6 +583,22 @@ def test_gemm_swiglu_fused_equals_separate(dtype, M, I, K):
     torch.testing.assert_close(got.float().cpu(), plain.swiglu(gu.cpu(), dtype), **tol(dtype))
 
 
+def test_pull_reads_and_keeps_nothing():
+    """The measurements' yardstick: reads a buffer of any length once (the tail of the last 16 KB included) and
+    writes nothing."""
+    from vosti_amd.kernels.ops import KernelError
+    k = kern(torch.bfloat16)
+    sink = torch.full((1,), 7, dtype=torch.int32, device="cuda")
+    for n in (8, 8200, 1 << 20, (1 << 20) + 24):
+        t = torch.randn(n, device="cuda").to(torch.bfloat16)
+        before = t.clone()
+        k.pull(t, sink)
+        torch.cuda.synchronize()
+        assert torch.equal(t, before) and sink.item() == 7
+    with pytest.raises(KernelError, match="contiguous"):
+        k.pull(torch.zeros(8, 8, device="cuda", dtype=torch.bfloat16)[:, :4], sink)
+
+
 def test_attention_rounds_probabilities_as_the_reference_does():
     """bfloat16: P is rounded to the element type for P.V while the normaliser sums the unrounded P
     (kernels/triton_kernels/fattn_paged.py:236-244).  On inputs where the rounding errors add up the

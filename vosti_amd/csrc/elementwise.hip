@@ -230,6 +230,27 @@ __global__ void fill_random_kernel(elem_t* __restrict__ out, int64_t n, uint64_t
   out[i] = from_f32<elem_t>(v);
 }
 
+// ------------------------------------------------------------- a yardstick
+// Reads `n16` 16-byte vectors and keeps nothing: every wave has 16 KB in flight and does nothing else.  What
+// this reaches on a buffer is what a kernel that must read that buffer once can reach at best; measurements
+// price the projections against it (bench.py).
+__global__ __launch_bounds__(512) void pull_kernel(const u32x4* __restrict__ p, int64_t n16, uint32_t* sink) {
+  const int lane = threadIdx.x & 63;
+  const int64_t wave = (int64_t)blockIdx.x * 8 + (threadIdx.x >> 6);
+  const int64_t first = wave * 1024;                   // this wave's 16 KB
+  if (first >= n16) return;
+  u32x4 v[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int64_t at = first + i * 64 + lane;
+    v[i] = p[at < n16 ? at : n16 - 1];                  // the last wave's tail: the last vector again
+  }
+  u32x4 a = v[0];
+#pragma unroll
+  for (int i = 1; i < 16; ++i) a ^= v[i];
+  if ((a.x ^ a.y ^ a.z ^ a.w) == 0x5a17c0deu && a.x == 0x12345678u) sink[0] = a.y;      // never, in practice: keeps the loads
+}
+
 // ================================================================ host side
 extern "C" {
 
@@ -327,6 +348,17 @@ int vk_rope_tables(elem_t* cos_t, elem_t* sin_t, const float* inv_freq, int max_
   const int64_t n = (int64_t)max_pos * half;
   rope_tables_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>(cos_t, sin_t, inv_freq, max_pos, half);
   return vk_check_launch("rope_tables");
+}
+
+// Reads `bytes` bytes at p (16-byte aligned) once and keeps nothing; `sink`: four bytes of device memory that are
+// practically never written.  For measurements only.
+int vk_pull(const void* p, int64_t bytes, void* sink, hipStream_t st) {
+  VK_REQUIRE(p != nullptr && sink != nullptr && ((uintptr_t)p % 16) == 0 && bytes >= 16, "pull: bad operands");
+  const int64_t n16 = bytes / 16;
+  const int64_t waves = (n16 + 1023) / 1024;
+  VK_REQUIRE((waves + 7) / 8 <= 0x7fffffff, "pull: buffer too large");
+  pull_kernel<<<(unsigned)((waves + 7) / 8), 512, 0, st>>>(static_cast<const u32x4*>(p), n16, static_cast<uint32_t*>(sink));
+  return vk_check_launch("pull");
 }
 
 int vk_fill_random(elem_t* out, int64_t n, uint64_t seed, int kind, float p0, float p1, hipStream_t st) {

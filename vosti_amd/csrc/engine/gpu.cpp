@@ -99,7 +99,7 @@ struct Kernels::Fn {
   int (*attn_item_rows)();
 };
 
-static constexpr int KERNEL_ABI = 12;
+static constexpr int KERNEL_ABI = 13;
 
 Kernels::Kernels(const std::string& lib_dir, const std::string& name) : name_(name), fn_(new Fn) {
   if (name == "bf16") dtype_ = DType::BF16;

@@ -29,6 +29,6 @@ int vk_elem_bytes(void) { return VK_ELEM_BYTES; }
 
 // Bumped whenever an exported signature changes; the Python side refuses a
 // library whose number differs from its own.
-int vk_abi_version(void) { return 12; }
+int vk_abi_version(void) { return 13; }
 
 }  // extern "C"

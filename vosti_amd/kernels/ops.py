@@ -15,7 +15,7 @@ import torch
 
 from . import build
 
-ABI_VERSION = 12
+ABI_VERSION = 13
 SEGMENT_KEYS = 256
 ATTN_ITEM_ROWS = 128      # rows of one prompt item of paged_attention
 
@@ -65,6 +65,7 @@ class Kernels:
         _sig(lib.vk_cast_from_f32, P, P, L, P)
         _sig(lib.vk_rope_tables, P, P, P, I, I, P)
         _sig(lib.vk_fill_random, P, L, c_uint64, I, F, F, P)
+        _sig(lib.vk_pull, P, L, P, P)
         _sig(lib.vk_gemm, P, P, P, I, I, I, L, L, I, P)
         _sig(lib.vk_gemm_swiglu, P, P, P, I, I, I, L, L, P)
         _sig(lib.vk_gemm_swiglu_supported, I, I, I)
@@ -195,6 +196,13 @@ class Kernels:
         self._call(self.lib.vk_rope_tables, cos.data_ptr(), sin.data_ptr(), self._f32(inv_freq, "inv_freq", half),
                    max_pos, half, self._stream())
         return cos, sin
+
+    def pull(self, t: torch.Tensor, sink: torch.Tensor) -> None:
+        """Reads ``t`` (contiguous) once and keeps nothing: the yardstick of what a kernel that must read it can
+        reach.  ``sink``: an int32 tensor on the GPU that is practically never written."""
+        if not t.is_contiguous() or not t.is_cuda:
+            raise KernelError("pull: a contiguous tensor on the GPU is needed")
+        self._call(self.lib.vk_pull, t.data_ptr(), t.numel() * t.element_size(), self._i32(sink, "sink"), self._stream())
 
     def fill_random(self, out: torch.Tensor, seed: int, kind: int, p0: float, p1: float) -> None:
         self._call(self.lib.vk_fill_random, self._elem(out, "out"), out.numel(), c_uint64(seed & (2**64 - 1)), kind,
