@@ -161,7 +161,7 @@ def main() -> int:
         torch.cuda.empty_cache()
         return dt / steps, ctx
 
-    def prefill_run(reps: int = 3):
+    def prefill_run(reps: int = 6):
         times = []
         for i in range(reps + 1):
             eng = Engine(model, num_pages=pages_per_request, page_size=page, max_num_seqs=1, max_num_batched_tokens=PROMPT_TOKENS,
