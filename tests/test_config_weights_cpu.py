@@ -71,7 +71,7 @@ def test_model_spec_is_data():
     m = spec.layers[1].mixer
     assert m.kind == "attention" and m.params["num_kv_heads"] == 2 and m.params["q_norm"].params["eps"] == 1e-5
     assert spec.layers[2].names["mixer.q_norm.weight"] == "model.layers.2.self_attn.q_norm.weight"
-    assert spec.head.params["tied"] is False
+    assert not spec.head.params["tied"]
 
 
 def test_load_config_errors(tmp_path):

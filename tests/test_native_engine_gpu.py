@@ -3,8 +3,7 @@
 Both engines drive the same kernels, cache manager and scheduler; what differs is everything between:
 configuration, weight loading, parts, step layout, graph replay, sampling state.  So the native engine's
 tokens must be the Python engine's, token for token, and pass the same checks against the plain
-implementation.  (The two compute the rotary frequencies with different pow routines, which may differ
-in the last bit of a frequency; the checks against the plain implementation hold for each alone.)"""
+implementation, and its logits bit for bit (every rule that both need is computed in one place)."""
 import json
 import os
 import shutil
@@ -17,6 +16,7 @@ from safetensors.torch import load_file, save_file
 from conftest import TINY
 from plain_qwen3 import PlainQwen3
 from test_engine_gpu import DTYPES, check_greedy_against_plain, engine, prompts
+from test_model_gpu import plain_logits  # noqa: F401  (a fixture)
 from vosti_amd.kernels import build
 
 pytestmark = pytest.mark.gpu
@@ -284,19 +284,24 @@ class _NativeRunner:
 
 @pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B", "C"])
-def test_every_cutting_through_the_native_step_function(tiny_dirs, name, dtype_name):
+def test_every_cutting_through_the_native_step_function(tiny_dirs, plain_logits, name, dtype_name):
     """The native engine's step function under the four cuttings of the Python one's test: every request alone
     and whole; all but the last 32 tokens in one step and the rest one by one; portions of changing size down to
-    one token; up to four live requests mixed, on so few pages that they are used again.  The logits of every
-    (request, position) are the same bits under all four, and the whole prompts' are the Python step function's
-    (where a rotation frequency differs in its last bit between the two pow routines, within that bit's reach)."""
-    from test_model_gpu import cut_chunks, cut_mixed, cut_tail, cut_whole, make_runner, prompts_for, replay, LENGTHS
+    one token; up to four live requests mixed, on so few pages that they are used again.  The whole prompts'
+    logits are the plain implementation's within what the type costs, the logits of every (request, position)
+    are the same bits under all four cuttings, and they are the bits of the Python step function."""
+    from test_model_gpu import (LENGTHS, assert_matches_plain, cut_chunks, cut_mixed, cut_tail, cut_whole, make_runner, prompts_for,
+                                replay)
     prompts = prompts_for(name)
     page = TINY[name][1]
+    ref, exact = plain_logits(name, dtype_name), plain_logits(name, "float32")
     mixed_steps, mixed_pages = cut_mixed(prompts, page)
     pages = -(-max(LENGTHS[name]) // page)
     runner = _NativeRunner(tiny_dirs[name], dtype_name, page, pages)
     whole = replay(runner, cut_whole(prompts))
+    for i, p in enumerate(prompts):
+        got = torch.stack([whole[(i, j)] for j in range(len(p))])
+        assert_matches_plain(got, ref[i], exact[i], dtype_name, f"request {i} (length {len(p)}), whole, native step function")
     for label, steps, n in (("tail", cut_tail(prompts), None), ("chunks", cut_chunks(prompts), None), ("mixed", mixed_steps, mixed_pages)):
         if n is not None:
             runner = _NativeRunner(tiny_dirs[name], dtype_name, page, n)
@@ -306,9 +311,37 @@ def test_every_cutting_through_the_native_step_function(tiny_dirs, name, dtype_n
         assert not bad, f"{label}: first differing (request, position) {bad[:1]} of {len(bad)}"
     py = replay(make_runner(tiny_dirs[name], dtype_name, page, num_pages=pages), cut_whole(prompts))
     differing = [k for k in sorted(whole) if not torch.equal(py[k], whole[k])]
-    if differing:
-        worst = max((py[k] - whole[k]).abs().max().item() for k in differing)
-        assert worst < (2e-2 if dtype_name == "bfloat16" else 1e-4), (len(differing), worst)
+    assert not differing, f"the two step functions differ at {differing[:1]} and {len(differing) - 1} more places"
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_replayed_steps_through_the_step_function_alone(tiny_dirs, dtype_name):
+    """The step function alone with recorded decode steps: four requests decode together (eagerly, recorded, then
+    replayed), and between the replays one of them decodes alone, a step that runs eagerly and leaves the
+    activation memory's cursor far below the recording's results.  The 32-bit copy of a replayed step's logits
+    must not be placed on top of them: every step's logits are those of an engine that replays nothing."""
+    from vosti_amd.engine import NativeEngine
+    ps = prompts("B", [9, 30, 17, 5], seed=12)
+    got = {}
+    for graphs in (False, True):
+        e = NativeEngine(tiny_dirs["B"], dtype=dtype_name, num_pages=64, page_size=8, max_num_seqs=8, enable_prefix_cache=False, graphs=graphs)
+        out = [e.trace_step([(i, p, [len(p) - 1]) for i, p in enumerate(ps)])]
+        tok = 7
+        for round_ in range(4):
+            for _ in range(3):                                       # all four rows: eager, recorded, replayed, ...
+                out.append(e.trace_step([(i, [tok + i], [0]) for i in range(4)]))
+                tok += 4
+            alone = round_ % 4
+            out.append(e.trace_step([(alone, [tok], [0])]))          # fewer rows, eagerly at first sight
+            tok += 1
+        if graphs:
+            assert e.stats()["graph_stats"]["replayed"] >= 8
+        for i in range(4):
+            e.trace_finish(i)
+        assert e.cache_check() == ""
+        got[graphs] = out
+    for a, b in zip(got[False], got[True]):
+        assert a.shape == b.shape and (a.view("<u4") == b.view("<u4")).all()
 
 
 FAMILY_WIDTHS = {       # hidden, inside, q heads, kv heads (head size 128): the layer sizes of the family's models

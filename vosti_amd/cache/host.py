@@ -1,12 +1,14 @@
-"""Loads the native host library (cache manager and scheduler)."""
+"""Loads the native host library: the cache manager, the scheduler, the architectures' reading of config.json
+and the rules that the native engine and this package share (rotation frequencies, the sizes that decode
+steps are recorded with)."""
 from __future__ import annotations
 
 import ctypes
-from ctypes import POINTER, c_char_p, c_int, c_int32, c_int64, c_uint64, c_void_p
+from ctypes import POINTER, c_char_p, c_double, c_int, c_int32, c_int64, c_uint64, c_void_p
 
 from ..kernels import build
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 _LIB = None
 
 
@@ -59,8 +61,68 @@ def host_lib():
     sig("vh_sched_num_running", I, P)
     sig("vh_sched_preemptions", c_int64, P)
     sig("vh_sched_is_live", I, P, U)
+    sig("vh_describe_config", I, c_char_p, c_char_p, I, c_char_p, I)
+    sig("vh_model_types", I, c_char_p, I)
+    sig("vh_rotary_inverse_frequencies", None, c_double, I, c_void_p)
+    sig("vh_graph_row_bucket", I, I)
+    sig("vh_graph_width_bucket", I, I)
+    sig("vh_max_graphs", I)
     _LIB = lib
     return lib
+
+
+class UnknownArchitecture(ValueError):
+    pass
+
+
+def describe_config(raw: dict) -> dict:
+    """What the native library's architecture makes of a config.json: the model's description as data
+    (``model_spec_json`` in csrc/host/spec.h) with the typed configuration under "config".  ValueError with the
+    library's text for a configuration that breaks a rule, UnknownArchitecture if the library has no such
+    architecture."""
+    import json
+    lib = host_lib()
+    text = json.dumps(raw).encode()
+    err = ctypes.create_string_buffer(2048)
+    cap = 1 << 16
+    while True:
+        out = ctypes.create_string_buffer(cap)
+        n = lib.vh_describe_config(text, out, cap, err, len(err))
+        if n == -2:
+            raise UnknownArchitecture(err.value.decode(errors="replace"))
+        if n < 0:
+            raise ValueError(err.value.decode(errors="replace"))
+        if n < cap:
+            return json.loads(out.value.decode())
+        cap = n + 1
+
+
+def native_model_types() -> dict[str, str]:
+    """model_type -> architecture name of every architecture the native library has."""
+    lib = host_lib()
+    out = ctypes.create_string_buffer(4096)
+    lib.vh_model_types(out, len(out))
+    return dict(line.split("=", 1) for line in out.value.decode().splitlines() if line)
+
+
+def rotary_inverse_frequencies(theta: float, rotary_dim: int):
+    """float32 numpy array [rotary_dim / 2]: 1 / theta^(2j / rotary_dim), the one routine every host uses."""
+    import numpy as np
+    out = np.empty(rotary_dim // 2, dtype=np.float32)
+    host_lib().vh_rotary_inverse_frequencies(float(theta), int(rotary_dim), out.ctypes.data)
+    return out
+
+
+def graph_row_bucket(rows: int) -> int:
+    return host_lib().vh_graph_row_bucket(int(rows))
+
+
+def graph_width_bucket(pages: int) -> int:
+    return host_lib().vh_graph_width_bucket(int(pages))
+
+
+def max_graphs() -> int:
+    return host_lib().vh_max_graphs()
 
 
 def i32_array(values):

@@ -70,6 +70,14 @@ class Arena {
  public:
   void* take(size_t bytes);
   void reset() { block_ = 0; offset_ = 0; }
+  // Where the next block would be handed out.  A recorded step's results lie below the mark taken at the end
+  // of its recording; after a replay the cursor goes back there, so that what is taken next (a copy of the
+  // logits, say) cannot lie on top of them.
+  struct Mark {
+    size_t block = 0, offset = 0;
+  };
+  Mark mark() const { return {block_, offset_}; }
+  void restore(const Mark& m) { block_ = m.block; offset_ = m.offset; }
   void forbid_growth(bool on) { frozen_ = on; }
   size_t capacity() const;
 

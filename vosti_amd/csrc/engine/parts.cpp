@@ -1,5 +1,7 @@
 #include "parts.h"
 
+#include "../host/rules.h"
+
 #include <cmath>
 #include <mutex>
 
@@ -99,8 +101,9 @@ class RMSNorm : public Norm {
 
 // Half-rotation rotary encoding with tables (python/vosti_kernels/rotary.py:80-90 for the frequencies,
 // :137-160 for the tables, kernels/triton_kernels/rope.py:78-123 for the rotation).  inv_freq[j] =
-// 1 / theta^(2j / rotary_dim) is computed once on the host in 32-bit; the angles, cosines and sines of
-// every position are computed on the GPU in 32-bit and stored as elements.
+// 1 / theta^(2j / rotary_dim) is computed once on the host in 32-bit (rotary_inverse_frequencies, the one
+// routine every host of these kernels uses); the angles, cosines and sines of every position are computed on
+// the GPU in 32-bit and stored as elements.
 class Rotary : public PositionEncoding {
  public:
   Rotary(const PartSpec& s, Kernels& k)
@@ -123,10 +126,7 @@ class Rotary : public PositionEncoding {
     if (it == shared.end()) {
       const int64_t half = rotary_dim_ / 2;
       std::vector<float> inv(half);
-      for (int64_t j = 0; j < half; ++j) {
-        const float exponent = (float)(2 * j) / (float)rotary_dim_;
-        inv[j] = 1.0f / std::pow((float)theta_, exponent);
-      }
+      rotary_inverse_frequencies(theta_, (int)rotary_dim_, inv.data());
       DeviceBuffer inv_dev(half * sizeof(float));
       hip_check(hipMemcpy(inv_dev.data(), inv.data(), half * sizeof(float), hipMemcpyHostToDevice), "rotary frequencies");
       Tensor inv_t;

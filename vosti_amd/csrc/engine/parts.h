@@ -12,7 +12,7 @@
 #include <vector>
 
 #include "gpu.h"
-#include "spec.h"
+#include "../host/spec.h"
 
 namespace vosti {
 

@@ -1,5 +1,7 @@
 #include "runner.h"
 
+#include "../host/rules.h"
+
 #include <algorithm>
 #include <cstring>
 
@@ -60,19 +62,6 @@ CachePool::CachePool(DecoderModel& model, int page_size_, int num_pages, int num
 }
 
 // ----------------------------------------------------------------------------------------- runner
-// Recorded decode steps have one of these numbers of rows; a step with fewer is filled up with rows that read
-// one key of page 0 and write nothing (the reference pads its graphs likewise,
-// python/vosti_kernels/graph_overlay.py:177-389).  Block tables are recorded with one of these widths times
-// eight pages, so that a long generation walks through few recordings.
-static int bucket(int n) {      // the smallest of 1, 2, 3, 4, 6, 8, 12, 16, ... that is at least n
-  for (int b = 1;; b *= 2) {
-    if (b >= n) return b;
-    if (b >= 2 && b + b / 2 >= n) return b + b / 2;
-  }
-}
-int ModelRunner::row_bucket(int rows) { return rows > 512 ? rows : bucket(rows); }
-int ModelRunner::width_bucket(int pages) { return 8 * bucket((std::max(pages, 1) + 7) / 8); }
-
 struct ModelRunner::Captured {
   hipGraph_t graph = nullptr;
   hipGraphExec_t exec = nullptr;
@@ -80,6 +69,7 @@ struct ModelRunner::Captured {
   std::unique_ptr<DeviceBuffer> meta;        // the device buffer the graph reads
   size_t ints = 0;
   Tensor logits;                             // the graph's output
+  Arena::Mark arena_end;                     // the arena's cursor when the recording ended
   hipEvent_t copied = nullptr;               // the last upload from `staging`
   std::shared_ptr<DeviceBuffer> workspace;   // the buffer its launches point into
   std::list<Key>::iterator lru_it;
@@ -324,6 +314,7 @@ ModelRunner::Captured* ModelRunner::capture(const Key& key, Layout& lay) {
   try {
     hip_check(begun, "begin of the recording");
     cap->logits = forward(lay, meta);
+    cap->arena_end = k_.arena.mark();
     hip_check(hipStreamEndCapture(k_.stream, &cap->graph), "end of the recording");
   } catch (...) {
     if (begun == hipSuccess && !cap->graph) {
@@ -349,9 +340,9 @@ ModelRunner::Captured* ModelRunner::capture(const Key& key, Layout& lay) {
 Tensor ModelRunner::run_decode_graph(const std::vector<StepEntry>& entries) {
   if (!poisoned_.empty()) throw GraphError("graph replay is switched off after a failure: " + poisoned_);
   std::vector<int> widths = needed_widths(entries);
-  for (int& w : widths) w = width_bucket(w);
+  for (int& w : widths) w = graph_width_bucket(w);
   // A mixer with state of its own would have to be told which rows are padding: no padding then.
-  const int rows = pool_.has_state ? (int)entries.size() : row_bucket((int)entries.size());
+  const int rows = pool_.has_state ? (int)entries.size() : graph_row_bucket((int)entries.size());
   const Key key{rows, widths};
   auto it = captured_.find(key);
   if (it == captured_.end() && seen_.insert(key).second) return run_eager(entries);   // first sight of a signature
@@ -373,6 +364,9 @@ Tensor ModelRunner::run_decode_graph(const std::vector<StepEntry>& entries) {
     }
     hip_check(hipEventRecord(cap->copied, k_.stream), "event record");
     hip_check(hipGraphLaunch(cap->exec, k_.stream), "graph launch");
+    // No forward() ran, so the arena's cursor is wherever the last eager step left it, which may be in the
+    // middle of this recording's results.
+    k_.arena.restore(cap->arena_end);
     logits = cap->logits.rows(0, (int64_t)entries.size());
   } catch (const std::exception& e) {
     poisoned_ = e.what();

@@ -20,6 +20,7 @@
 #include <vector>
 
 #include "../host/cache_manager.h"
+#include "../host/rules.h"
 #include "model.h"
 
 namespace vosti {
@@ -60,7 +61,7 @@ struct GraphStats {
 
 class ModelRunner {
  public:
-  ModelRunner(DecoderModel& model, CachePool& pool, bool graphs, int max_graphs = 24);
+  ModelRunner(DecoderModel& model, CachePool& pool, bool graphs, int max_graphs = kMaxGraphs);
   ~ModelRunner();
 
   // The forward pass of a step whose pages are taken; logits [wanted, vocab] in the element type, valid
@@ -70,8 +71,6 @@ class ModelRunner {
   Tensor step(const std::vector<StepEntry>& entries);
   void finish(RequestId id);
   const GraphStats& graph_stats() const { return stats_; }
-  static int width_bucket(int pages);
-  static int row_bucket(int rows);
 
  private:
   struct Piece {

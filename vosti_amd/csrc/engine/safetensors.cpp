@@ -13,22 +13,9 @@
 #include <sstream>
 
 #include "gpu.h"
-#include "json.h"
+#include "../host/json.h"
 
 namespace vosti {
-
-std::string read_text_file(const std::string& path) {
-  std::ifstream f(path, std::ios::binary);
-  if (!f) throw EngineError("cannot read " + path);
-  std::ostringstream s;
-  s << f.rdbuf();
-  return s.str();
-}
-
-bool file_exists(const std::string& path) {
-  struct stat st;
-  return stat(path.c_str(), &st) == 0 && S_ISREG(st.st_mode);
-}
 
 static std::string real_path(const std::string& p) {
   char buf[PATH_MAX];
@@ -72,7 +59,10 @@ void Checkpoint::map_file(const std::string& path) {
   const int fd = open(path.c_str(), O_RDONLY);
   if (fd < 0) throw EngineError("cannot open " + path);
   struct stat st;
-  fstat(fd, &st);
+  if (fstat(fd, &st) != 0 || st.st_size < 0) {
+    close(fd);
+    throw EngineError("cannot read the size of " + path);
+  }
   const size_t size = (size_t)st.st_size;
   if (size < 8) {
     close(fd);
@@ -94,16 +84,24 @@ void Checkpoint::map_file(const std::string& path) {
     if (!dt || !sh || !off || off->items.size() != 2) throw EngineError(path + ": malformed entry for " + m.first);
     StoredTensor t;
     t.dtype = dt->text;
-    int64_t n = 1;
+    // The header's numbers are the file's word, not ours: a negative or overflowing one must not become a
+    // pointer outside the mapping.
+    const uint64_t limit = (uint64_t)1 << 56;
+    uint64_t n = 1;
     for (const Json& s : sh->items) {
-      t.shape.push_back(s.as_int());
-      n *= s.as_int();
+      if (!s.is_int() || s.as_int() < 0) throw EngineError(path + ": " + m.first + " has a shape entry that is no size");
+      const uint64_t d = (uint64_t)s.as_int();
+      if (d != 0 && n > limit / d) throw EngineError(path + ": the shape of " + m.first + " is larger than any file");
+      t.shape.push_back((int64_t)d);
+      n *= d;
     }
+    if (!off->items[0].is_int() || !off->items[1].is_int() || off->items[0].as_int() < 0 || off->items[1].as_int() < 0)
+      throw EngineError(path + ": " + m.first + " has data offsets that are no sizes");
     const size_t b = (size_t)off->items[0].as_int(), e = (size_t)off->items[1].as_int();
-    if (e < b || data_start + e > size) throw EngineError(path + ": " + m.first + " lies outside the file");
+    if (e < b || e > size - data_start) throw EngineError(path + ": " + m.first + " lies outside the file");
     auto it = stored_sizes().find(t.dtype);
-    if (it != stored_sizes().end() && (size_t)n * it->second != e - b)
-      throw EngineError(path + ": " + m.first + " has " + std::to_string(e - b) + " bytes, its shape needs " + std::to_string((size_t)n * it->second));
+    if (it != stored_sizes().end() && n * (uint64_t)it->second != (uint64_t)(e - b))
+      throw EngineError(path + ": " + m.first + " has " + std::to_string(e - b) + " bytes, its shape needs " + std::to_string(n * (uint64_t)it->second));
     t.data = p + data_start + b;
     t.bytes = e - b;
     t.file = path;

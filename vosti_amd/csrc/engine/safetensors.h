@@ -9,6 +9,8 @@
 #include <string>
 #include <vector>
 
+#include "../host/files.h"
+
 namespace vosti {
 
 struct StoredTensor {
@@ -37,8 +39,5 @@ class Checkpoint {
   std::vector<Mapping> maps_;
   std::map<std::string, StoredTensor> entries_;
 };
-
-std::string read_text_file(const std::string& path);
-bool file_exists(const std::string& path);
 
 }  // namespace vosti

@@ -4,7 +4,9 @@
 #include <vector>
 
 #include "cache_manager.h"
+#include "rules.h"
 #include "scheduler.h"
+#include "spec.h"
 
 using namespace vosti;
 
@@ -20,7 +22,7 @@ struct SchedulerHandle {
 
 extern "C" {
 
-int vh_abi_version(void) { return 7; }
+int vh_abi_version(void) { return 8; }
 
 // ------------------------------------------------------------ cache manager
 void* vh_cache_create(int page_size, int n_groups, const int* windows, const int* num_pages, int num_slots,
@@ -157,5 +159,51 @@ int vh_sched_num_running(void* h) { return SH->sched.num_running(); }
 int64_t vh_sched_preemptions(void* h) { return SH->sched.preemptions(); }
 int vh_sched_is_live(void* h, uint64_t id) { return SH->sched.is_live(id) ? 1 : 0; }
 #undef SH
+
+// ------------------------------------------------- configurations and shared rules
+// What the architecture named by a config.json's text makes of it: model_spec_json().  Returns the text's
+// length (the caller's buffer got it whole if that is below cap), or -1 with the reason in err; -2 if no
+// registered architecture is named (err says which are).
+int vh_describe_config(const char* config_text, char* out, int cap, char* err, int errcap) {
+  auto fail = [&](const std::string& what, int rc) {
+    if (err && errcap > 0) {
+      std::strncpy(err, what.c_str(), (size_t)errcap - 1);
+      err[errcap - 1] = 0;
+    }
+    return rc;
+  };
+  try {
+    register_builtin_architectures();
+    const Json raw = Json::parse(config_text);
+    if (!architecture_known(raw)) {
+      try {
+        model_spec_from_config(raw);
+      } catch (const std::exception& e) {
+        return fail(e.what(), -2);
+      }
+    }
+    const std::string text = model_spec_json(model_spec_from_config(raw));
+    if ((int)text.size() < cap) std::memcpy(out, text.c_str(), text.size() + 1);
+    return (int)text.size();
+  } catch (const JsonError& e) {
+    return fail(std::string("config.json is not valid JSON: ") + e.what(), -1);
+  } catch (const std::exception& e) {
+    return fail(e.what(), -1);
+  }
+}
+
+// "model_type=Architecture" lines of every registered architecture.
+int vh_model_types(char* out, int cap) {
+  register_builtin_architectures();
+  std::string text;
+  for (const auto& t : model_types()) text += t.first + "=" + t.second + "\n";
+  if ((int)text.size() < cap) std::memcpy(out, text.c_str(), text.size() + 1);
+  return (int)text.size();
+}
+
+void vh_rotary_inverse_frequencies(double theta, int rotary_dim, float* out) { rotary_inverse_frequencies(theta, rotary_dim, out); }
+int vh_graph_row_bucket(int rows) { return graph_row_bucket(rows); }
+int vh_graph_width_bucket(int pages) { return graph_width_bucket(pages); }
+int vh_max_graphs(void) { return kMaxGraphs; }
 
 }  // extern "C"

@@ -7,7 +7,7 @@
 // geometry is admitted and both are parameters.
 #include <cmath>
 
-#include "spec.h"
+#include "qwen3.h"
 
 namespace vosti {
 namespace {
@@ -50,9 +50,9 @@ PartSpecPtr part(std::string kind, std::map<std::string, double> numbers, std::m
   return p;
 }
 
-// Pre-norm blocks of attention and SwiGLU (src/exec/dense_swiglu_decoder.rs:43-441), every layer alike,
-// run once each in order (src/exec/dense_swiglu_model.rs:131-1041).
-ModelSpec qwen3(const Json& raw) {
+}  // namespace
+
+Qwen3Config qwen3_config(const Json& raw) {
   if (const Json* mt = present(raw, "model_type"))
     if (mt->text != "qwen3") throw ConfigError("config.json: 'model_type' is '" + mt->text + "', expected 'qwen3'");
   const int64_t hidden = pos_int(raw, "hidden_size");
@@ -103,12 +103,37 @@ ModelSpec qwen3(const Json& raw) {
   const int64_t layers = nl->as_int();
   if (layer_types && (int64_t)layer_types->items.size() != layers)
     throw ConfigError("config.json: 'layer_types' must have one entry per layer");
-  const int64_t vocab = pos_int(raw, "vocab_size");
-  const int64_t inter = pos_int(raw, "intermediate_size");
-  const int64_t max_pos = pos_int(raw, "max_position_embeddings");
-  const double eps = pos_float(present(raw, "rms_norm_eps"), "rms_norm_eps");
-  const double rope_theta = pos_float(theta, "rope_theta");
+  Qwen3Config c;
+  c.vocab_size = pos_int(raw, "vocab_size");
+  c.hidden_size = hidden;
+  c.intermediate_size = pos_int(raw, "intermediate_size");
+  c.num_hidden_layers = layers;
+  c.num_attention_heads = heads;
+  c.num_key_value_heads = kv_heads;
+  c.head_dim = head_dim;
+  c.max_position_embeddings = pos_int(raw, "max_position_embeddings");
+  c.rms_norm_eps = pos_float(present(raw, "rms_norm_eps"), "rms_norm_eps");
+  c.rope_theta = pos_float(theta, "rope_theta");
+  c.tie_word_embeddings = tie;
+  return c;
+}
 
+std::string Qwen3Config::to_json() const {
+  return "{\"vocab_size\": " + std::to_string(vocab_size) + ", \"hidden_size\": " + std::to_string(hidden_size) +
+         ", \"intermediate_size\": " + std::to_string(intermediate_size) + ", \"num_hidden_layers\": " + std::to_string(num_hidden_layers) +
+         ", \"num_attention_heads\": " + std::to_string(num_attention_heads) + ", \"num_key_value_heads\": " + std::to_string(num_key_value_heads) +
+         ", \"head_dim\": " + std::to_string(head_dim) + ", \"max_position_embeddings\": " + std::to_string(max_position_embeddings) +
+         ", \"rms_norm_eps\": " + json_number(rms_norm_eps) + ", \"rope_theta\": " + json_number(rope_theta) +
+         ", \"tie_word_embeddings\": " + (tie_word_embeddings ? "true" : "false") + "}";
+}
+
+// Pre-norm blocks of attention and SwiGLU (src/exec/dense_swiglu_decoder.rs:43-441), every layer alike,
+// run once each in order (src/exec/dense_swiglu_model.rs:131-1041).
+ModelSpec qwen3_model_spec(const Qwen3Config& c) {
+  const int64_t hidden = c.hidden_size, heads = c.num_attention_heads, kv_heads = c.num_key_value_heads, head_dim = c.head_dim;
+  const int64_t vocab = c.vocab_size, inter = c.intermediate_size, max_pos = c.max_position_embeddings, layers = c.num_hidden_layers;
+  const double eps = c.rms_norm_eps, rope_theta = c.rope_theta;
+  const bool tie = c.tie_word_embeddings;
   const PartSpecPtr norm = part("rmsnorm", {{"size", (double)hidden}, {"eps", eps}});
   const PartSpecPtr head_norm = part("rmsnorm", {{"size", (double)head_dim}, {"eps", eps}});
   const PartSpecPtr rope = part("rotary", {{"head_dim", (double)head_dim}, {"rotary_dim", (double)head_dim}, {"theta", rope_theta},
@@ -154,16 +179,15 @@ ModelSpec qwen3(const Json& raw) {
                 {"final_norm.weight", "model.norm.weight"},
                 {"head.weight", tie ? "model.embed_tokens.weight" : "lm_head.weight"}};
   if (tie) spec.ignored_names = {"lm_head.weight"};
+  spec.config_json = c.to_json();
   return spec;
 }
-
-}  // namespace
 
 void register_builtin_architectures() {
   static bool done = false;
   if (done) return;
   done = true;
-  register_architecture("Qwen3ForCausalLM", "qwen3", qwen3);
+  register_architecture("Qwen3ForCausalLM", "qwen3", [](const Json& raw) { return qwen3_model_spec(qwen3_config(raw)); });
 }
 
 }  // namespace vosti

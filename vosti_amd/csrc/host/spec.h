@@ -54,8 +54,19 @@ struct ModelSpec {
   std::vector<ScheduleEntry> schedule;
   std::map<std::string, std::string> names;          // "embedding.weight", "final_norm.weight", "head.weight"
   std::vector<std::string> ignored_names;            // tensors a checkpoint may hold although the model does not use them
+  std::string config_json = "{}";                    // the typed configuration the architecture read, as a JSON object
   void validate() const;
 };
+
+// A number as JSON writes it: whole numbers without a fraction, others with the 17 digits that give the
+// same 64-bit value back.
+std::string json_number(double v);
+std::string json_string(const std::string& s);
+// The description as one JSON object: {"architecture", "vocab_size", "hidden_size", "max_positions", "config",
+// "embedding", "final_norm", "head" (parts: {"kind", "numbers", "parts"}), "layers" ([{"block", "mixer",
+// "feed_forward", "norms", "names"}]), "schedule" ([[layer, cache_from]]), "names", "ignored_names"}.  Hosts in
+// other languages read the rules of an architecture from this instead of writing them again.
+std::string model_spec_json(const ModelSpec& spec);
 
 using ArchitectureFactory = std::function<ModelSpec(const Json& config)>;
 void register_architecture(const std::string& name, const std::string& model_type, ArchitectureFactory make);
@@ -64,6 +75,8 @@ std::map<std::string, std::string> model_types();
 // Reads DIR/config.json, finds the architecture by its "architectures" entry and returns its description.
 ModelSpec model_spec_from_dir(const std::string& model_dir);
 ModelSpec model_spec_from_config(const Json& config);
+// Whether the configuration names an architecture of this registry (by "architectures", else by "model_type").
+bool architecture_known(const Json& config);
 // Registers the architectures that are built into this program; safe to call more than once.
 void register_builtin_architectures();
 

@@ -23,29 +23,16 @@ import numpy as np
 import torch
 
 from ..cache import CachePool
+from ..cache.host import graph_row_bucket, graph_width_bucket, max_graphs as _max_graphs
 from ..parts.base import GroupTables, HostStep, StepContext
 
-# Captured decode steps have one of these numbers of rows; a step with fewer is filled up with rows that
-# read one key of page 0 and write nothing (the reference pads its graphs likewise,
-# python/vosti_kernels/graph_overlay.py:177-389).  Block tables are captured with one of these widths
-# times eight pages, so that a long generation walks through few captures.
-ROW_BUCKETS = (1, 2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64, 96, 128, 192, 256, 384, 512)
-WIDTH_STEP = 8
-MAX_GRAPHS = 24        # captured graphs kept; the least recently replayed one goes first
-
-
-def _bucket(n: int) -> int:
-    """The smallest of 1, 2, 3, 4, 6, 8, 12, 16, ... that is at least n."""
-    b = 1
-    while True:
-        for m in (b, b + b // 2):
-            if m >= n and (m == b or b >= 2):
-                return m
-        b *= 2
-
-
-def width_bucket(pages: int) -> int:
-    return WIDTH_STEP * _bucket(-(-max(pages, 1) // WIDTH_STEP))
+# Captured decode steps have one of the numbers of rows 1, 2, 3, 4, 6, 8, 12, 16, ...; a step with fewer is filled
+# up with rows that read one key of page 0 and write nothing (the reference pads its graphs likewise,
+# python/vosti_kernels/graph_overlay.py:177-389).  Block tables are captured with one of these numbers times
+# eight pages, so that a long generation walks through few captures.  The numbers, and how many graphs are
+# kept, are the native library's (csrc/host/rules.h), which the native engine's step function uses too.
+row_bucket = graph_row_bucket
+width_bucket = graph_width_bucket
 
 
 class GraphError(RuntimeError):
@@ -90,11 +77,11 @@ class _Captured:
 class ModelRunner:
     """Binds a model to a cache pool and runs steps."""
 
-    def __init__(self, model, pool: CachePool, graphs: bool = False, max_graphs: int = MAX_GRAPHS):
+    def __init__(self, model, pool: CachePool, graphs: bool = False, max_graphs: int | None = None):
         self.model, self.pool, self.cache = model, pool, pool.manager
         self.kernels = model.kernels
         self.graphs = graphs
-        self.max_graphs = max(1, int(max_graphs))
+        self.max_graphs = max(1, int(_max_graphs() if max_graphs is None else max_graphs))   # the least recently replayed goes first
         self._workspace: torch.Tensor | None = None
         self._seen: set[tuple] = set()
         self._captured: "OrderedDict[tuple, _Captured]" = OrderedDict()
@@ -262,7 +249,7 @@ class ModelRunner:
         P = self.pool.page_size
         widths = [width_bucket(w) for w in self.needed_widths(entries)]
         # A mixer with state of its own would have to be told which rows are padding: no padding then.
-        rows = len(entries) if self.pool.has_state else next((b for b in ROW_BUCKETS if b >= len(entries)), len(entries))
+        rows = len(entries) if self.pool.has_state else row_bucket(len(entries))
         key = (rows, tuple(widths))
         cap = self._captured.get(key)
         if cap is None and key not in self._seen:

@@ -4,7 +4,8 @@ Three shared libraries and one program are built from ``vosti_amd/csrc``:
 
 * ``libvosti_bf16.so`` and ``libvosti_f32.so``: the gfx950 kernels, the same
   sources compiled with ``-DVK_BF16`` or ``-DVK_F32`` (hipcc);
-* ``libvosti_host.so``: the cache manager and the scheduler (g++, no GPU code);
+* ``libvosti_host.so``: the cache manager, the scheduler, the architectures' reading of config.json and
+  the rules that every host of the kernels shares (g++, no GPU code);
 * ``vosti_engine``: the native engine and its command line (``csrc/engine`` with
   the cache manager and the scheduler compiled in; g++ against the HIP runtime;
   it loads the kernel library of the chosen precision from its own folder), and
@@ -93,7 +94,9 @@ def _sources(name: str) -> tuple[list[Path], list[Path]]:
     if name in ("engine", "engine_lib"):
         engine = CSRC / "engine"
         face = "capi.cpp" if name == "engine" else "main.cpp"       # the file of the other face is left out
-        return ([p for p in sorted(engine.glob("*.cpp")) if p.name != face] + [host / "cache_manager.cpp", host / "scheduler.cpp"],
+        # Everything of the host library but its C interface and the plain references of the kernels.
+        shared = [p for p in sorted(host.glob("*.cpp")) if p.name not in ("capi.cpp", "reference.cpp")]
+        return ([p for p in sorted(engine.glob("*.cpp")) if p.name != face] + shared,
                 sorted(engine.glob("*.h")) + sorted(host.glob("*.h")))
     return sorted(CSRC.glob("*.hip")), sorted(CSRC.glob("*.h"))
 

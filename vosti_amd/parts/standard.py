@@ -10,6 +10,7 @@ from typing import Mapping
 import numpy as np
 import torch
 
+from ..cache.host import rotary_inverse_frequencies
 from ..config.spec import PartSpec
 from ..kernels.ops import ATTN_ITEM_ROWS, Kernels, SEGMENT_KEYS
 from .base import (Block, Embedding, FeedForward, Head, HostStep, KVPagesSpec, Mixer, Norm, PagedKV, ParamSpec, Part,
@@ -68,8 +69,9 @@ class Rotary(PositionEncoding):
     tables, kernels/triton_kernels/rope.py:78-123 for the rotation).
 
     inv_freq[j] = 1 / theta^(2j / rotary_dim) is computed once on the host in
-    fp32, exactly as the reference writes it; the angles, cosines and sines of
-    every position are computed on the GPU in fp32 and stored as elements."""
+    fp32 by the native library's routine (csrc/host/rules.h), which the native
+    engine calls too, so that both have the same bits; the angles, cosines and
+    sines of every position are computed on the GPU in fp32 and stored as elements."""
 
     def __init__(self, kernels: Kernels, head_dim: int, rotary_dim: int, theta: float, max_positions: int):
         super().__init__(kernels)
@@ -82,8 +84,7 @@ class Rotary(PositionEncoding):
         if self._tables is None:
             key = (self.kernels.name, self.rotary_dim, self.theta, self.max_positions, torch.cuda.current_device())
             if key not in _ROTARY_TABLES:
-                exponent = torch.arange(0, self.rotary_dim, 2, dtype=torch.int64).to(torch.float32) / self.rotary_dim
-                inv_freq = (1.0 / (self.theta ** exponent)).to("cuda")
+                inv_freq = torch.from_numpy(rotary_inverse_frequencies(self.theta, self.rotary_dim)).to("cuda")
                 _ROTARY_TABLES[key] = self.kernels.rope_tables(inv_freq, self.max_positions)
             self._tables = _ROTARY_TABLES[key]
         return self._tables
