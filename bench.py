@@ -9,9 +9,13 @@
 A step is one decode step of the engine (plan, forward, sample, commit) for a
 batch of B requests whose prompts of 2,048 random tokens were prefilled through
 the same engine.  One JSON line is printed: ``value`` is decoded tokens per
-second; ``prefill`` times one 2,048-token prompt; ``roofline`` prices the decode
-step's compulsory HBM reads (every weight once, the live requests' cache)
-against 8 TB/s; ``points`` holds decode throughput at batch 1 and 64.
+second; ``prefill`` times one 2,048-token prompt (the median of six; the best is
+beside it); ``roofline`` prices the decode step's compulsory HBM reads (every
+weight once, the live requests' cache) against 8 TB/s; ``points`` holds decode
+throughput at batch 1 and 64 and, unless --no-other-shapes, the figures of the
+two larger workloads.  Every figure is measured through the engine that
+``config.engine`` names (the native one unless --engine python); the one point
+measured through the other engine says so in its name.
 """
 from __future__ import annotations
 
@@ -77,12 +81,13 @@ def main() -> int:
     ap.add_argument("--graphs", type=int, default=1, choices=[0, 1], help="replay decode steps from captured HIP graphs")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill timing")
     ap.add_argument("--no-per-kernel", action="store_true", help="skip the timing of the dominant kernels on their own")
+    ap.add_argument("--no-other-shapes", action="store_true", help="skip the 14B and 32B workloads that the default record holds as points")
     ap.add_argument("--prompt-tokens", type=int, default=PROMPT_TOKENS,
                     help="context length of the decode measurement (the prefill figure is always of 2,048 tokens)")
     ap.add_argument("--workload", default="decode8b", choices=["decode8b", "mixed14b", "prefix32b"])
     ap.add_argument("--engine", default="native", choices=["native", "python"],
-                    help="which engine runs the timed decode steps: the native one (vosti_amd.engine.NativeEngine, the same "
-                         "kernels, cache manager and scheduler without Python between two steps) or the Python one")
+                    help="which engine every figure is measured through: the native one (vosti_amd.engine.NativeEngine) or the "
+                         "Python step function over the same kernels, cache manager and scheduler")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -100,7 +105,8 @@ def main() -> int:
     from vosti_amd.weights import random_weights_on_gpu
 
     if args.workload != "decode8b":
-        return other_workload(args)
+        print(json.dumps(other_workload(args)), flush=True)
+        return 0
     if args.batch is None:
         args.batch = 8
     shape = QWEN3_SHAPES[args.shape]
@@ -108,8 +114,11 @@ def main() -> int:
     if args.layers is None:
         args.layers = shape["num_hidden_layers"]
     cfg = Qwen3Config(**dict(shape, num_hidden_layers=args.layers))
-    model = build_model(cfg, args.dtype)
-    random_weights_on_gpu(model, seed=0)
+    # The Python package's model: for the Python engine, and for timing the kernels on their own with its weights.
+    need_model = args.engine == "python" or not args.no_points or not args.no_per_kernel
+    model = build_model(cfg, args.dtype) if need_model else None
+    if model is not None:
+        random_weights_on_gpu(model, seed=0)
     torch.cuda.synchronize()
     elem = 2 if args.dtype == "bfloat16" else 4
     dt_name = "bf16" if args.dtype == "bfloat16" else "fp32"
@@ -162,19 +171,26 @@ def main() -> int:
         return dt / steps, ctx
 
     def prefill_run(reps: int = 6):
+        """Seconds for one prompt of 2,048 tokens to its first token, through the engine: every run of one engine (the
+        first, untimed, loads the kernels), each a new request on pages that the one before gave back."""
+        kw = dict(num_pages=pages_per_request, page_size=page, max_num_seqs=1, max_num_batched_tokens=PROMPT_TOKENS,
+                  enable_prefix_cache=False)
+        if args.engine == "native":
+            eng = NativeEngine(native_dir.name, dtype=args.dtype, random_weights_seed=0, **kw)
+        else:
+            eng = Engine(model, **kw)
         times = []
         for i in range(reps + 1):
-            eng = Engine(model, num_pages=pages_per_request, page_size=page, max_num_seqs=1, max_num_batched_tokens=PROMPT_TOKENS,
-                         enable_prefix_cache=False)
             eng.add_request(prompt(PROMPT_TOKENS), SamplingParams(max_tokens=1))
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             out = eng.step()
             torch.cuda.synchronize()
             times.append(time.perf_counter() - t0)
-            assert len(out) == 1
-            del eng
-        return min(times[1:])
+            assert len(out) == 1 and not eng.has_unfinished()
+        del eng
+        torch.cuda.empty_cache()
+        return sorted(times[1:])
 
     kernels: dict = {}
     step_s, ctx = decode_run(args.batch, args.steps, args.warmup, None if args.no_per_kernel else kernels)
@@ -196,15 +212,18 @@ def main() -> int:
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
     }
     if not args.no_points:
-        t = prefill_run()
+        times = prefill_run()
+        t = (times[len(times) // 2 - 1] + times[len(times) // 2]) / 2 if len(times) % 2 == 0 else times[len(times) // 2]
         flops = prefill_flops(cfg, PROMPT_TOKENS)
         record["prefill"] = {"value": round(PROMPT_TOKENS / t, 1), "tokens": PROMPT_TOKENS, "ms": round(t * 1e3, 3),
-                             "frac": round(flops / t / PEAK_FLOPS[dt_name], 4)}
+                             "frac": round(flops / t / PEAK_FLOPS[dt_name], 4), "of": "median of six", "best_ms": round(times[0] * 1e3, 3),
+                             "engine": args.engine}
         points = {}
-        # 48 untimed steps first: at batch 1 the first forty or so steps after a new engine's prompt run 4 % slower
-        # than the rest (4.35 against 4.18 ms), whichever engine runs them.
-        for B, name in ((1, "decode_b1"), (64, "decode_b64")):
-            s, _ = decode_run(B, min(args.steps, 32), max(args.warmup, 48))
+        # At batch 1 the first forty or so steps after a new engine's prompt run 4 % slower than the rest (4.35 against
+        # 4.18 ms), whichever engine runs them: the point is taken after 48 untimed steps, and the steps right after
+        # the prompt and those after 150 steps stand beside it.
+        for B, name, warm in ((1, "decode_b1", 48), (1, "decode_b1_first_steps", 2), (1, "decode_b1_after_150_steps", 150), (64, "decode_b64", 48)):
+            s, _ = decode_run(B, min(args.steps, 32), max(args.warmup, warm) if warm >= 48 else warm)
             points[name] = round(B / s, 2)
         # The same steps through the other engine: what the Python host code between two steps costs.
         other = "python" if args.engine == "native" else "native"
@@ -220,6 +239,24 @@ def main() -> int:
                 kernels["prefill"] = {"error": f"{type(e).__name__}: {e}"}
     if kernels:
         record["kernels"] = kernels
+    if not args.no_points and not args.no_other_shapes and args.shape == "8b" and args.dtype == "bfloat16":
+        # The two larger workloads of the same family, whole models, as points of this record (their own records:
+        # --workload mixed14b, --workload prefix32b).
+        del model
+        torch.cuda.empty_cache()
+        for workload in ("mixed14b", "prefix32b"):
+            other_args = argparse.Namespace(**dict(vars(args), workload=workload, layers=None, batch=None, steps=16, warmup=8))
+            try:
+                r = other_workload(other_args)
+            except Exception as e:          # the record's own figures stand without these
+                record["points"][workload + "_error"] = f"{type(e).__name__}: {e}"
+                continue
+            if workload == "mixed14b":
+                record["points"].update(mixed14b_tokens_per_s=r["value"], mixed14b_output_tokens_per_s=r["output"]["value"],
+                                        mixed14b_wall_s=r["output"]["wall_s"])
+            else:
+                record["points"].update(prefix32b_decode_b64_tokens_per_s=r["value"], prefix32b_ms_per_step=r["ms_per_step"],
+                                        prefix32b_roofline_frac=r["roofline"]["frac"], prefix32b_prefill_tokens_per_s=r["prefill"]["value"])
     print(json.dumps(record), flush=True)
     return 0
 
@@ -326,8 +363,8 @@ def progress(text: str, state={"t": 0.0}) -> None:
         print(f"bench.py: {text}", file=sys.stderr, flush=True)
 
 
-def other_workload(args) -> int:
-    """The two larger shapes with the workloads named for them: one JSON line each, same fields."""
+def other_workload(args) -> dict:
+    """The two larger shapes with the workloads named for them: a record each, same fields."""
     import torch
     from vosti_amd.config import Qwen3Config
     import tempfile
@@ -340,11 +377,17 @@ def other_workload(args) -> int:
     full_layers = shape["num_hidden_layers"]
     layers = args.layers if args.layers is not None else full_layers
     cfg = Qwen3Config(**dict(shape, num_hidden_layers=layers))
-    print(f"bench.py: {args.workload}: building {layers} layers", file=sys.stderr, flush=True)
-    model = build_model(cfg, args.dtype)
-    random_weights_on_gpu(model, seed=0)
-    torch.cuda.synchronize()
-    print("bench.py: weights ready", file=sys.stderr, flush=True)
+    print(f"bench.py: {args.workload}: building {layers} layers for the {args.engine} engine", file=sys.stderr, flush=True)
+    native_dir = tempfile.TemporaryDirectory()          # what the native engine is given: config.json; it draws the weights itself
+    with open(os.path.join(native_dir.name, "config.json"), "w") as f:
+        json.dump(cfg.to_dict(), f)
+
+    def make_engine(**kw):
+        if args.engine == "native":
+            return NativeEngine(native_dir.name, dtype=args.dtype, random_weights_seed=0, **kw)
+        model = build_model(cfg, args.dtype)
+        random_weights_on_gpu(model, seed=0)
+        return Engine(model, **kw)
     elem = 2 if args.dtype == "bfloat16" else 4
     dt_name = "bf16" if args.dtype == "bfloat16" else "fp32"
     rng = random.Random(1)
@@ -355,7 +398,7 @@ def other_workload(args) -> int:
     shape_keys = {"model": name, "layers": layers, "layers_of_model": full_layers, "hidden_size": cfg.hidden_size,
                   "intermediate_size": cfg.intermediate_size, "q_heads": cfg.num_attention_heads,
                   "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim, "vocab_size": cfg.vocab_size,
-                  "page_size": page, "parallelism": "single GPU", "graphs": bool(args.graphs)}
+                  "page_size": page, "parallelism": "single GPU", "graphs": bool(args.graphs), "engine": args.engine}
 
     if args.workload == "mixed14b":
         # 32 prompts of 128 to 4,096 tokens, 128 new tokens each; prompts enter in portions of at most 4,096
@@ -364,8 +407,10 @@ def other_workload(args) -> int:
         lengths = [rng.randint(128, 4096) for _ in range(n)]
         prompts = [[rng.randrange(cfg.vocab_size) for _ in range(L)] for L in lengths]
         pages = sum(-(-(L + new + 1) // page) for L in lengths) + 8
-        eng = Engine(model, num_pages=pages, page_size=page, max_num_seqs=n, max_num_batched_tokens=4096,
-                     enable_prefix_cache=False, graphs=bool(args.graphs))
+        eng = make_engine(num_pages=pages, page_size=page, max_num_seqs=n, max_num_batched_tokens=4096,
+                          enable_prefix_cache=False, graphs=bool(args.graphs))
+        torch.cuda.synchronize()
+        print("bench.py: weights ready", file=sys.stderr, flush=True)
         sp = SamplingParams(max_tokens=new, ignore_eos=True)
         for p_ in prompts:
             eng.add_request(p_, sp)
@@ -387,8 +432,7 @@ def other_workload(args) -> int:
                       output={"value": round(emitted / dt, 1), "wall_s": round(dt, 3)},
                       roofline={"bound": "mfma", "achieved": round(flops / dt / 1e12, 1), "peak": PEAK_FLOPS[dt_name] / 1e12,
                                 "unit": "TFLOP/s (projections only)", "frac": round(flops / dt / PEAK_FLOPS[dt_name], 4)})
-        print(json.dumps(record), flush=True)
-        return 0
+        return record
 
     # prefix32b: 64 requests whose prompts share their first 1,024 tokens and go on with 7,168 of their own;
     # the pages of the shared part are computed once and reused.  Decode steps are timed at context ~8,200.
@@ -398,44 +442,51 @@ def other_workload(args) -> int:
     # The first requests decode while the later ones are still prefilled, one a step: room for that too.
     total = args.steps + args.warmup + n + 16
     pages = shared_len // page + n * (-(-(own_len + total + 1) // page)) + 8
-    eng = Engine(model, num_pages=pages, page_size=page, max_num_seqs=n, max_num_batched_tokens=8192,
-                 enable_prefix_cache=True, graphs=bool(args.graphs))
+    eng = make_engine(num_pages=pages, page_size=page, max_num_seqs=n, max_num_batched_tokens=8192,
+                      enable_prefix_cache=True, graphs=bool(args.graphs))
+    torch.cuda.synchronize()
+    print("bench.py: weights ready", file=sys.stderr, flush=True)
     sp = SamplingParams(max_tokens=total, ignore_eos=True)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     # The first request alone, so that its pages are published before the others look for them.
     eng.add_request(prompts[0], sp)
-    eng.step()
+    emitted_tokens = len(eng.step())
     for p_ in prompts[1:]:
         eng.add_request(p_, sp)
-    while eng.scheduler.num_waiting() or any(eng.cache.length(r) < shared_len + own_len for r in range(n)):
-        eng.step()
-        progress(f"prefill: {eng.scheduler.num_waiting()} requests waiting")
+    while True:                                             # until every request has its first token: all of them decode
+        out = eng.step()
+        emitted_tokens += len(out)
+        progress(f"prefill: {len(out)} requests decoding")
+        if len(out) == n:
+            break
     torch.cuda.synchronize()
     prefill_s = time.perf_counter() - t0
     print(f"bench.py: prefill done in {prefill_s:.1f} s", file=sys.stderr, flush=True)
     for _ in range(args.warmup):
         assert len(eng.step()) == n
+    emitted_tokens += args.warmup * n
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
         eng.step()
     torch.cuda.synchronize()
     step_s = (time.perf_counter() - t0) / args.steps
-    ctx = sum(eng.cache.length(r) for r in range(n)) / n - (args.steps - 1) / 2.0     # mean keys a request reads in a timed step
+    # Mean keys a request reads in a timed step: its prompt, the tokens it had put out before, and the steps so far.
+    ctx = shared_len + own_len + emitted_tokens / n + (args.steps - 1) / 2.0
+    prefix_hits = eng.stats()["prefix_hits"] if args.engine == "native" else eng.cache.prefix_hits()
     layers_w, head_w = gemm_params(cfg)
     kv_token = 2 * cfg.num_key_value_heads * cfg.head_dim * cfg.num_hidden_layers
     unique = (layers_w + head_w + (n * (ctx - shared_len) + shared_len) * kv_token) * elem     # shared pages once
     record = dict(base, metric=f"decode tok/s at batch {n}, context 8,192, a 1,024-token prefix shared through the page cache, Qwen3-32B shape",
                   value=round(n / step_s, 1), steps=args.steps, warmup=args.warmup, ms_per_step=round(step_s * 1e3, 3),
                   config=dict(shape_keys, global_batch=n, seq_len=shared_len + own_len + total, shared_prefix=shared_len,
-                              context_at_timing=round(ctx), reused_prefix_pages=eng.cache.prefix_hits()),
+                              context_at_timing=round(ctx), reused_prefix_pages=prefix_hits),
                   prefill={"value": round((n * own_len + shared_len) / prefill_s, 1), "tokens": n * own_len + shared_len,
                            "ms": round(prefill_s * 1e3, 1)},
                   roofline={"bound": "hbm", "achieved": round(unique / step_s / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                             "frac": round(unique / step_s / 1e9 / HBM_PEAK_GBS, 4)})
-    print(json.dumps(record), flush=True)
-    return 0
+    return record
 
 
 if __name__ == "__main__":

@@ -16,7 +16,7 @@ def host_lib():
     global _LIB
     if _LIB is not None:
         return _LIB
-    lib = ctypes.CDLL(str(build.ensure("host")))
+    lib = ctypes.CDLL(str(build.ensure("host")), mode=ctypes.RTLD_GLOBAL)     # global: plugins of the native engine register with it
     lib.vh_abi_version.restype = c_int
     if lib.vh_abi_version() != ABI_VERSION:
         raise RuntimeError("libvosti_host.so is stale; rebuild it")

@@ -17,7 +17,32 @@ void put(char* err, int cap, const std::string& text) {
 
 extern "C" {
 
-int ve_abi_version(void) { return 2; }
+int ve_abi_version(void) { return 3; }
+
+// Loads a shared library of part kinds and architectures (load_plugin in parts.h).  0, or -1 with the reason.
+int ve_load_plugin(const char* path, char* err, int errcap) {
+  try {
+    load_plugin(path);
+    return 0;
+  } catch (const std::exception& e) {
+    put(err, errcap, e.what());
+    return -1;
+  }
+}
+
+// 1 if this library can run the model in the folder; 0 if its architecture or one of its part kinds is not
+// registered here (err says which); -1 if config.json is missing or breaks a rule (err says how).
+int ve_supports(const char* model_dir, char* err, int errcap) {
+  try {
+    const std::string why = why_unsupported(model_dir);
+    if (why.empty()) return 1;
+    put(err, errcap, why);
+    return 0;
+  } catch (const std::exception& e) {
+    put(err, errcap, e.what());
+    return -1;
+  }
+}
 
 // dtype: "bf16" or "f32".  random_weights != 0: the folder needs config.json only and the weights are drawn
 // from `seed` on the GPU.

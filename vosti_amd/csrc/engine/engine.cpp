@@ -20,9 +20,30 @@ float uniform_for(uint64_t seed, uint64_t output_index) {
 static const char* ADMISSION[] = {"Accepted", "DuplicateRequestId", "EmptyPrompt", "TooManyEosTokenIds", "ZeroMaxTokens",
                                   "HistoryCapacityOverflow", "EmptyEosTokenIds"};
 
+std::string why_unsupported(const std::string& model_dir) {
+  register_builtin_architectures();
+  register_standard_parts();
+  const std::string path = model_dir + "/config.json";
+  if (!file_exists(path)) throw ConfigError(path + " is missing");
+  Json raw;
+  try {
+    raw = Json::parse(read_text_file(path));
+  } catch (const JsonError& e) {
+    throw ConfigError(path + ": " + e.what());
+  }
+  if (!architecture_known(raw)) {
+    const Json* archs = raw.get("architectures");
+    const std::string name = (archs && archs->kind == Json::Array && !archs->items.empty()) ? archs->items[0].text : "";
+    return "architecture '" + name + "' is not registered in the native engine";
+  }
+  const std::string missing = missing_part(model_spec_from_config(raw));
+  return missing.empty() ? "" : "the native engine has no " + missing;
+}
+
 Engine::Engine(const EngineOptions& opt) {
   register_builtin_architectures();
   register_standard_parts();
+  for (const std::string& p : opt.plugins) load_plugin(p);
   int devices = 0;
   hip_check(hipGetDeviceCount(&devices), "looking for a GPU");
   if (devices < 1) throw EngineError("no GPU: this engine has no CPU path");
@@ -143,6 +164,16 @@ std::vector<int32_t> Engine::forward_and_sample(const std::vector<PlanRow>& rows
   const int R = (int)sampling.size();
   if (R == 0) return sampled;
   if (R > sample_rows_) throw EngineError("more sampled rows than the engine was made for");
+  if (observer_.active()) {
+    const Tensor f = kernels_->to_f32(logits);
+    observed_.resize((size_t)f.numel());
+    hip_check(hipMemcpyAsync(observed_.data(), f.data, f.bytes(), hipMemcpyDeviceToHost, kernels_->stream), "logits readback");
+    hip_check(hipStreamSynchronize(kernels_->stream), "logits readback");
+    std::vector<int> places;
+    for (size_t i = 0; i < rows.size(); ++i)
+      if (rows[i].sample) places.push_back((int)i);
+    observer_.rows(observed_.data(), logits.dim(1), places, steps_, dtype_name(kernels_->dtype()));
+  }
   bool any_temperature = false;
   for (int i = 0; i < R; ++i) {
     const PlanRow& r = *sampling[i];

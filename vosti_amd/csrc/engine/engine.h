@@ -13,6 +13,7 @@
 #include <vector>
 
 #include "../host/scheduler.h"
+#include "observe.h"
 #include "runner.h"
 
 namespace vosti {
@@ -45,7 +46,12 @@ struct EngineOptions {
   bool graphs = false;           // VOSTI_CUDA_GRAPH (engine_setup.rs:79-81)
   bool random_weights = false;   // draw the weights from random_seed on the GPU; the folder needs config.json only
   uint64_t random_seed = 0;
+  std::vector<std::string> plugins;    // shared libraries with part kinds and architectures of their own (load_plugin)
 };
+
+// Why this engine cannot run the model in the folder, or "" if it can: an architecture that is not registered,
+// or a part kind that its description names and no registered part has.  Configuration errors are thrown.
+std::string why_unsupported(const std::string& model_dir);
 
 // What one engine step took, for measurements.
 struct StepTime {
@@ -74,6 +80,10 @@ class Engine {
   ModelRunner& runner() { return *runner_; }
   DecoderModel& model() { return *model_; }
   const std::vector<RequestId>& last_scheduled() const { return last_scheduled_; }
+  // Requests added from now on get ids from `id` on (never below what was given out already): the reference's
+  // drivers give every workload of one engine a base of its own (examples/support/engine_calls.rs:70-118).
+  void set_next_request_id(RequestId id) { next_id_ = std::max(next_id_, id); }
+  int page_size() const { return pool_->page_size; }
   void record_step_times(bool on) { record_times_ = on; }
   const std::vector<StepTime>& step_times() const { return step_times_; }
 
@@ -96,6 +106,10 @@ class Engine {
   std::vector<RequestId> last_scheduled_;
   bool record_times_ = false;
   std::vector<StepTime> step_times_;
+  // VOSTI_LOGITS_DIGEST / VOSTI_LOGITS_OBSERVER_DIR: hashes or copies of every sampled logits row, to compare runs
+  // that batch differently (python/vosti_kernels/kernels.py:1020-1033).
+  LogitsObserver observer_;
+  std::vector<float> observed_;
   // The sampler's buffers: temperatures and uniform numbers up, token ids down.
   float* sample_in_ = nullptr;        // pinned [2, rows]
   int32_t* sample_out_ = nullptr;     // pinned [rows]

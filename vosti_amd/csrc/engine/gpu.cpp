@@ -226,6 +226,26 @@ Tensor Kernels::to_f32(const Tensor& x) {
   return out;
 }
 
+void Kernels::copy_columns(Tensor& dst, int64_t dst_first, const Tensor& src, int64_t src_first, int64_t count) {
+  if (src.shape.size() != 2 || dst.shape.size() != 2 || src.dim(0) != dst.dim(0) || src.dtype != dst.dtype || count < 0 || src_first < 0 ||
+      dst_first < 0 || src_first + count > src.dim(1) || dst_first + count > dst.dim(1))
+    throw EngineError("copy_columns: " + std::to_string(count) + " columns from " + std::to_string(src_first) + " of " + src.describe() +
+                      " to " + std::to_string(dst_first) + " of " + dst.describe());
+  if (count == 0 || src.dim(0) == 0) return;
+  const size_t e = (size_t)dtype_bytes(src.dtype);
+  hip_check(hipMemcpy2DAsync(static_cast<char*>(dst.data) + (size_t)dst_first * e, (size_t)dst.dim(1) * e,
+                             static_cast<const char*>(src.data) + (size_t)src_first * e, (size_t)src.dim(1) * e, (size_t)count * e,
+                             (size_t)src.dim(0), hipMemcpyDeviceToDevice, stream),
+            "copying columns");
+}
+
+Tensor Kernels::columns(const Tensor& x, int64_t first, int64_t count) {
+  if (x.shape.size() != 2) throw EngineError("columns of " + x.describe());
+  Tensor out = empty({x.dim(0), count}, x.dtype);
+  copy_columns(out, 0, x, first, count);
+  return out;
+}
+
 void Kernels::rope_tables(Tensor& cos, Tensor& sin, const Tensor& inv_freq) {
   const int64_t half = inv_freq.numel();
   expect(inv_freq, "inverse frequencies", DType::F32, {half});

@@ -109,6 +109,10 @@ class Kernels {
   Tensor swiglu(const Tensor& gate_up);
   Tensor gather_rows(const Tensor& x, const Tensor& rows);
   Tensor to_f32(const Tensor& x);
+  // Columns [first, first + count) of a [rows, width] tensor as a tensor of their own.
+  Tensor columns(const Tensor& x, int64_t first, int64_t count);
+  // dst[:, dst_first : dst_first + count] = src[:, src_first : src_first + count], rows alike.
+  void copy_columns(Tensor& dst, int64_t dst_first, const Tensor& src, int64_t src_first, int64_t count);
   void rope_tables(Tensor& cos, Tensor& sin, const Tensor& inv_freq);
   // Counter-based random fill: element i is a function of (seed, i); kind 0: a sum of four 16-bit uniforms
   // scaled by p0, kind 1: p0 + u * p1.

@@ -20,6 +20,12 @@
 //     VOSTI_OUTPUT_TOKENS        --output-tokens       write "index<TAB>ids" lines to this file
 //     VOSTI_BENCH_INPUT          --bench-input         TSV of MAX_TOKENS<TAB>IDS[<TAB>ARRIVAL_STEP] requests
 //     VOSTI_BENCH_WARMUP_INPUT   --bench-warmup-input  a TSV of other requests, served first by the same engine
+//     VOSTI_BENCH_GRAPH_PRIMER_INPUT --bench-graph-primer-input  a third TSV, served before the warm-up so that the
+//                                                      recordings of its decode steps exist before anything is timed
+//     VOSTI_BENCH_CALLS          --bench-calls         JSON of several calls served one after the other by one engine
+//     VOSTI_BENCH_CALL_RESULTS   --bench-call-results  where their records go (a new JSON file)
+//     VOSTI_LOGITS_DIGEST                              a file that gets "row sha256" for every sampled logits row
+//     VOSTI_LOGITS_OBSERVER_DIR                        a folder that gets every sampled logits row as float32 .npy and an index
 //     VOSTI_MAX_MODEL_LEN        --max-model-len       longest prompt plus output (default: the model's positions)
 //     VOSTI_ENGINE_STEP_TRACE    --step-trace          append one JSON line per step to this file
 //
@@ -28,7 +34,9 @@
 // VOSTI_PREFIX_CACHE / --prefix-cache (0, 1), VOSTI_LIB_DIR / --lib-dir (where the kernel libraries lie;
 // default: beside this program), VOSTI_RANDOM_WEIGHTS / --random-weights SEED (the folder needs config.json
 // only; the weights are those of the Python launcher's random-model kind for that seed), VOSTI_STEP_TIMES /
-// --step-times FILE (one line "rows tokens sampled ms" per engine step).  End tokens come from generation_config.json's eos_token_id (one to three
+// --step-times FILE (one line "rows tokens sampled ms" per engine step), VOSTI_PLUGINS (paths, colon-separated) /
+// --plugin PATH (may be given more than once): shared libraries that register part kinds and architectures of
+// their own before the model folder is read.  End tokens come from generation_config.json's eos_token_id (one to three
 // ids: python/vosti_kernels/serving_workload.py:78-108); without that file there are none.  It prints
 // MODEL_OUTPUT_TOKEN_IDS=[...] like the reference, or a BENCH batch=... tok_s=... line for prepared requests.
 #include <unistd.h>
@@ -133,6 +141,15 @@ std::string id_list(const std::vector<int32_t>& ids, const char* sep) {
   return s;
 }
 
+std::vector<std::string> split_list(const std::string& text, char sep) {
+  std::vector<std::string> out;
+  std::stringstream ss(text);
+  std::string item;
+  while (std::getline(ss, item, sep))
+    if (!item.empty()) out.push_back(item);
+  return out;
+}
+
 struct Options {
   std::string kind = "engine", family;
   std::string model_path = env_or("MODEL_PATH", ""), device = env_or("CUDA_DEVICE", "cuda:0");
@@ -145,6 +162,8 @@ struct Options {
   long graphs = to_int(env_or("VOSTI_CUDA_GRAPH", "0"), "VOSTI_CUDA_GRAPH");
   std::string output_tokens = env_or("VOSTI_OUTPUT_TOKENS", ""), bench_input = env_or("VOSTI_BENCH_INPUT", "");
   std::string bench_warmup_input = env_or("VOSTI_BENCH_WARMUP_INPUT", "");
+  std::string bench_graph_primer_input = env_or("VOSTI_BENCH_GRAPH_PRIMER_INPUT", "");
+  std::string bench_calls = env_or("VOSTI_BENCH_CALLS", ""), bench_call_results = env_or("VOSTI_BENCH_CALL_RESULTS", "");
   long max_model_len = to_int(env_or("VOSTI_MAX_MODEL_LEN", "0"), "VOSTI_MAX_MODEL_LEN");
   std::string step_trace = env_or("VOSTI_ENGINE_STEP_TRACE", ""), dtype = env_or("VOSTI_DTYPE", "bfloat16");
   double temperature = std::atof(env_or("VOSTI_TEMPERATURE", "0").c_str());
@@ -153,6 +172,7 @@ struct Options {
   long prefix_cache = to_int(env_or("VOSTI_PREFIX_CACHE", "1"), "VOSTI_PREFIX_CACHE");
   std::string lib_dir = env_or("VOSTI_LIB_DIR", "");
   std::string random_weights = env_or("VOSTI_RANDOM_WEIGHTS", ""), step_times = env_or("VOSTI_STEP_TIMES", "");
+  std::vector<std::string> plugins = split_list(env_or("VOSTI_PLUGINS", ""), ':');
 };
 
 Options parse(int argc, char** argv) {
@@ -186,6 +206,9 @@ Options parse(int argc, char** argv) {
     else if (a == "--output-tokens") o.output_tokens = val();
     else if (a == "--bench-input") o.bench_input = val();
     else if (a == "--bench-warmup-input") o.bench_warmup_input = val();
+    else if (a == "--bench-graph-primer-input") o.bench_graph_primer_input = val();
+    else if (a == "--bench-calls") o.bench_calls = val();
+    else if (a == "--bench-call-results") o.bench_call_results = val();
     else if (a == "--max-model-len") o.max_model_len = to_int(val(), a);
     else if (a == "--step-trace") o.step_trace = val();
     else if (a == "--dtype") o.dtype = val();
@@ -196,6 +219,7 @@ Options parse(int argc, char** argv) {
     else if (a == "--lib-dir") o.lib_dir = val();
     else if (a == "--random-weights") o.random_weights = val();
     else if (a == "--step-times") o.step_times = val();
+    else if (a == "--plugin") o.plugins.push_back(val());
     else throw Usage("unknown option " + a);
   }
   return o;
@@ -254,8 +278,94 @@ int describe(const Options& o) {
   return 0;
 }
 
+std::string ids_json(const std::vector<std::vector<int32_t>>& lists) {
+  std::string s = "[";
+  for (size_t i = 0; i < lists.size(); ++i) s += (i ? ", [" : "[") + id_list(lists[i], ", ") + "]";
+  return s + "]";
+}
+
+// Several calls through one engine, one after the other (examples/support/engine_calls.rs:58-123):
+// {"prefix_caching": bool, "calls": [{"label", "prompts" | "output_prefix_from", "max_tokens"}]}.  A call's prompts
+// are given outright, or built from an earlier call's prompt, the first `count` tokens that call generated for it,
+// and a suffix (:32-56).  Without prefix caching the cached pages are dropped before every call.  One record per
+// call goes to the results file, and CALLS_FINISHED <n> is printed.
+int run_calls(Engine& engine, const Options& o, const std::vector<int32_t>& eos) {
+  const Json spec = Json::parse(read_text_file(o.bench_calls));
+  const Json* calls = spec.get("calls");
+  if (!calls || calls->kind != Json::Array || calls->items.empty()) throw Usage("bench calls: the file holds no calls");
+  if (o.bench_call_results.empty()) throw Usage("bench calls: VOSTI_BENCH_CALL_RESULTS (or --bench-call-results) is required");
+  if (file_exists(o.bench_call_results)) throw Usage("bench calls: " + o.bench_call_results + " exists already");
+  const Json* pc = spec.get("prefix_caching");
+  const bool prefix_caching = pc && pc->kind == Json::Bool && pc->boolean;
+  std::vector<std::pair<std::vector<std::vector<int32_t>>, std::vector<std::vector<int32_t>>>> prior;
+  std::string records = "[";
+  RequestId base = 0;
+  for (size_t index = 0; index < calls->items.size(); ++index) {
+    const Json& call = calls->items[index];
+    if (engine.has_unfinished()) throw Usage("bench calls: the call before did not finish");
+    const int dropped = prefix_caching ? 0 : engine.cache().drop_cached();
+    std::vector<std::vector<int32_t>> prompts;
+    if (const Json* src = call.get("output_prefix_from")) {
+      const Json *c = src->get("call"), *r = src->get("request"), *n = src->get("count");
+      if (!c || !r || !n) throw Usage("bench calls: 'output_prefix_from' needs 'call', 'request' and 'count'");
+      if (c->as_int() < 0 || c->as_int() >= (int64_t)prior.size()) throw Usage("bench calls: 'output_prefix_from' names a call that has not run yet");
+      const auto& from = prior[(size_t)c->as_int()];
+      if (r->as_int() < 0 || r->as_int() >= (int64_t)from.first.size()) throw Usage("bench calls: 'output_prefix_from' names a request that the call does not have");
+      const auto& out = from.second[(size_t)r->as_int()];
+      if (n->as_int() < 0 || n->as_int() > (int64_t)out.size()) throw Usage("bench calls: 'output_prefix_from' wants more tokens than were generated");
+      std::vector<int32_t> query = from.first[(size_t)r->as_int()];
+      query.insert(query.end(), out.begin(), out.begin() + n->as_int());
+      if (const Json* suffix = src->get("suffix"))
+        for (const Json& t : suffix->items) query.push_back((int32_t)t.as_int());
+      prompts.push_back(std::move(query));
+    } else if (const Json* ps = call.get("prompts")) {
+      for (const Json& p : ps->items) {
+        prompts.emplace_back();
+        for (const Json& t : p.items) prompts.back().push_back((int32_t)t.as_int());
+      }
+    }
+    const Json* mt = call.get("max_tokens");
+    const int max_tokens = mt ? (int)mt->as_int() : 0;
+    bool empty = prompts.empty() || max_tokens <= 0;
+    for (const auto& p : prompts) empty = empty || p.empty();
+    if (empty) throw Usage("bench calls: a call has an empty prompt, an empty batch or no output budget");
+    setenv("VOSTI_LOGITS_OBSERVER_PHASE", ("call-" + std::to_string(index)).c_str(), 1);
+    SamplingParams p;
+    p.max_tokens = max_tokens;
+    p.temperature = (float)o.temperature;
+    p.seed = (uint64_t)o.seed;
+    p.eos_token_ids = eos;
+    p.ignore_eos = o.ignore_eos;
+    engine.set_next_request_id(base);
+    engine.synchronize();
+    const auto t0 = std::chrono::steady_clock::now();
+    const auto outputs = engine.generate(prompts, {p});
+    const double wall = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+    const Json* label = call.get("label");
+    const GraphStats& g = engine.runner().graph_stats();
+    char wall_text[40];
+    std::snprintf(wall_text, sizeof wall_text, "%.9f", wall);
+    records += std::string(index ? ", " : "") + "{\"label\": " + json_string(label ? label->text : std::to_string(index)) +
+               ", \"request_id_base\": " + std::to_string(base) + ", \"input_token_ids\": " + ids_json(prompts) +
+               ", \"output_token_ids\": " + ids_json(outputs) + ", \"reclaimed_pages_before_call\": " + std::to_string(dropped) +
+               ", \"cache_isolated\": " + (prefix_caching ? "false" : "true") + ", \"cache_page_tokens\": " + std::to_string(engine.page_size()) +
+               ", \"wall_s\": " + wall_text + ", \"graph_stats\": {\"eager\": " + std::to_string(g.eager) + ", \"captured\": " +
+               std::to_string(g.captured) + ", \"replayed\": " + std::to_string(g.replayed) + ", \"evicted\": " + std::to_string(g.evicted) + "}}";
+    base += prompts.size();
+    prior.emplace_back(prompts, outputs);
+  }
+  records += "]";
+  std::FILE* f = std::fopen(o.bench_call_results.c_str(), "wx");
+  if (!f) throw Usage("bench calls: cannot create " + o.bench_call_results);
+  std::fputs(records.c_str(), f);
+  std::fclose(f);
+  std::cout << "CALLS_FINISHED " << calls->items.size() << "\n";
+  return 0;
+}
+
 int run(int argc, char** argv) {
   Options o = parse(argc, argv);
+  for (const std::string& p : o.plugins) load_plugin(p);
   if (o.kind == "describe") {
     if (o.model_path.empty()) throw Usage("MODEL_PATH (or --model-path) is required");
     return describe(o);
@@ -271,15 +381,21 @@ int run(int argc, char** argv) {
   if (o.graphs != 0 && o.graphs != 1) throw Usage("--graphs must be 0 or 1");
   if (o.prefix_cache != 0 && o.prefix_cache != 1) throw Usage("--prefix-cache must be 0 or 1");
   if (o.temperature < 0) throw Usage("--temperature must not be negative");
-  std::vector<Prepared> requests, warmup;
-  if (!o.bench_input.empty()) requests = parse_prepared(o.bench_input);
-  else requests.push_back({(int)o.max_tokens, parse_ids(o.prompt_ids), 0});
+  std::vector<Prepared> requests, warmup, primer;
+  if (!o.bench_calls.empty()) {
+  } else if (!o.bench_input.empty()) {
+    requests = parse_prepared(o.bench_input);
+  } else {
+    requests.push_back({(int)o.max_tokens, parse_ids(o.prompt_ids), 0});
+  }
   if (!o.bench_input.empty() && !o.bench_warmup_input.empty()) warmup = parse_prepared(o.bench_warmup_input);
+  if (!warmup.empty() && !o.bench_graph_primer_input.empty()) primer = parse_prepared(o.bench_graph_primer_input);
   const std::vector<int32_t> eos = eos_ids(o.model_path);
   eo.lib_dir = o.lib_dir.empty() ? self_dir() : o.lib_dir;
   eo.num_pages = (int)o.num_blocks;
   eo.page_size = (int)o.page_size;
-  eo.max_num_seqs = o.max_seqs > 0 ? (int)o.max_seqs : (int)std::max<size_t>({requests.size(), warmup.size(), (size_t)1});
+  eo.max_num_seqs = o.max_seqs > 0 ? (int)o.max_seqs
+                                   : (int)std::max<size_t>({requests.size(), warmup.size(), primer.size(), o.bench_calls.empty() ? (size_t)1 : (size_t)8});
   eo.max_num_batched_tokens = (int)o.max_batched_tokens;
   eo.prefix_cache = o.prefix_cache == 1;
   eo.max_model_len = (int)o.max_model_len;
@@ -300,7 +416,9 @@ int run(int argc, char** argv) {
     const std::string architecture = model_spec_from_dir(o.model_path).architecture;
     if (architecture != it->second) throw Usage(o.model_path + " holds a " + architecture + ", not a " + o.family + " model");
   }
+  eo.plugins = o.plugins;
   Engine engine(eo);
+  if (!o.bench_calls.empty()) return run_calls(engine, o, eos);
   engine.record_step_times(!o.step_times.empty());
   std::FILE* trace = nullptr;
   if (!o.step_trace.empty()) {
@@ -350,12 +468,20 @@ int run(int argc, char** argv) {
     return "{\"admitted_requests\":" + std::to_string(reqs.size()) + ",\"requests_with_reuse\":" + std::to_string(s.requests_with_reuse) +
            ",\"reused_prefix_blocks\":" + std::to_string(s.reused_blocks);
   };
+  if (!primer.empty()) {
+    // An optional third workload, served first in the same engine, so that the recordings of the decode steps it
+    // walks through exist before the warm-up (examples/support/engine_serving.rs:162-181).  Nothing is reported of it.
+    setenv("VOSTI_LOGITS_OBSERVER_PHASE", "primer", 1);
+    serve(primer, o.seed + (long)(requests.size() + warmup.size()));
+  }
   if (!warmup.empty()) {
     // The reference serves a disjoint warm-up workload in the same engine before the measured one
     // (examples/support/engine_serving.rs:157-206) and reports both (engine_benchmark.rs:45-76).
+    setenv("VOSTI_LOGITS_OBSERVER_PHASE", "warmup", 1);
     const Served w = serve(warmup, o.seed + (long)requests.size());
     std::cout << line("WARMUP", warmup, w, false) << "\n" << "WARMUP_CACHE_STATS " << stats(warmup, w) << "}\n";
   }
+  if (!warmup.empty()) setenv("VOSTI_LOGITS_OBSERVER_PHASE", "measured", 1);
   const Served s = serve(requests, o.seed);
   if (trace) std::fclose(trace);
   if (!o.step_times.empty()) {

@@ -2,6 +2,8 @@
 
 #include "../host/rules.h"
 
+#include <dlfcn.h>
+
 #include <cmath>
 #include <mutex>
 
@@ -23,6 +25,63 @@ void register_part(const std::string& category, const std::string& kind, PartFac
   part_registry()[{category, kind}] = std::move(make);
 }
 void register_block(const std::string& kind, BlockFactory make) { block_registry()[kind] = std::move(make); }
+bool part_registered(const std::string& category, const std::string& kind) { return part_registry().count({category, kind}) > 0; }
+bool block_registered(const std::string& kind) { return block_registry().count(kind) > 0; }
+
+namespace {
+std::string missing_in(const std::string& category, const PartSpec& p) {
+  if (!part_registered(category, p.kind)) return category + " part '" + p.kind + "'";
+  // Parts below a part: the name says the category ("q_norm", "k_norm": norms; "position").
+  for (const auto& c : p.parts) {
+    const std::string below = c.first == "position" ? "position" : (c.first.size() >= 4 && c.first.compare(c.first.size() - 4, 4, "norm") == 0 ? "norm" : "");
+    if (below.empty()) continue;
+    const std::string m = missing_in(below, *c.second);
+    if (!m.empty()) return m;
+  }
+  return "";
+}
+}  // namespace
+
+std::string missing_part(const ModelSpec& spec) {
+  std::string m = missing_in("embedding", *spec.embedding);
+  if (m.empty()) m = missing_in("norm", *spec.final_norm);
+  if (m.empty()) m = missing_in("head", *spec.head);
+  for (const LayerSpec& l : spec.layers) {
+    if (!m.empty()) break;
+    if (!block_registered(l.block)) m = "block arrangement '" + l.block + "'";
+    if (m.empty()) m = missing_in("mixer", *l.mixer);
+    if (m.empty()) m = missing_in("feed_forward", *l.feed_forward);
+    for (const auto& n : l.norms)
+      if (m.empty()) m = missing_in("norm", *n.second);
+  }
+  return m;
+}
+
+void load_plugin(const std::string& path) {
+  static std::mutex mutex;
+  static std::map<std::string, void*> loaded;
+  std::lock_guard<std::mutex> lock(mutex);
+  if (loaded.count(path)) return;
+  void* h = dlopen(path.c_str(), RTLD_NOW | RTLD_GLOBAL);
+  if (!h) throw EngineError("cannot load the plugin " + path + ": " + dlerror());
+  auto fn = reinterpret_cast<void (*)()>(dlsym(h, "vosti_plugin_register"));
+  if (!fn) throw EngineError("the plugin " + path + " has no vosti_plugin_register()");
+  register_standard_parts();
+  register_builtin_architectures();
+  fn();
+  loaded[path] = h;
+}
+
+std::pair<Tensor, Tensor> PositionEncoding::apply(const Tensor& q, const Tensor& k, const Tensor& positions) {
+  const Tensor *cos = cos_table(), *sin = sin_table();
+  if (!cos || !sin) throw EngineError("a position encoding needs tables of angles or an apply() of its own");
+  auto rotate = [&](const Tensor& x) {
+    if (x.shape.size() != 3) throw EngineError("position encoding of " + x.describe() + ", expected [tokens, heads, head size]");
+    const int64_t T = x.dim(0), n = x.dim(1), d = x.dim(2);
+    return kernels.qkv_post(x.view({T, n * d}), (int)n, 0, (int)d, nullptr, nullptr, 0, nullptr, nullptr, 0.f, cos, sin, &positions, nullptr);
+  };
+  return {rotate(q), k.data ? rotate(k) : Tensor()};
+}
 
 std::unique_ptr<Part> build_any_part(const std::string& category, const PartSpec& spec, Kernels& k) {
   auto it = part_registry().find({category, spec.kind});
@@ -162,8 +221,9 @@ struct AttentionItems {
 
 // Causal grouped-query attention over the paged cache (src/exec/dense_swiglu_decoder.rs:171-367): QKV
 // projection without bias, per-head norm of q and k, rotary encoding, store of k and v, attention, output
-// projection.  window > 0 limits a query to that many last keys.  Head norms and the rotation run inside
-// one launch, so the native engine takes norms that are a weighted row scale and rotations by table.
+// projection.  window > 0 limits a query to that many last keys.  q_norm, k_norm and position are parts of
+// their own; when they are weighted row scales and a rotation by tables the three steps between the projections
+// run as one launch.
 class Attention : public Mixer {
  public:
   Attention(const PartSpec& s, Kernels& k)
@@ -175,8 +235,6 @@ class Attention : public Mixer {
     if (const PartSpec* p = s.part("q_norm")) q_norm_ = build_part<Norm>("norm", *p, k);
     if (const PartSpec* p = s.part("k_norm")) k_norm_ = build_part<Norm>("norm", *p, k);
     if (const PartSpec* p = s.part("position")) position_ = build_part<PositionEncoding>("position", *p, k);
-    if (q_norm_ && k_norm_ && q_norm_->eps() != k_norm_->eps())
-      throw ConfigError("attention: the native engine runs the q and k norms in one launch and needs one eps for both");
   }
   std::vector<ParamDecl> params() const override {
     return {{"q_proj.weight", {(int64_t)nq_ * d_, hidden_}}, {"k_proj.weight", {(int64_t)nkv_ * d_, hidden_}},
@@ -194,9 +252,15 @@ class Attention : public Mixer {
     // weight are q's, then k's, then v's.
     w_qkv_ = stack_rows({need(t, "q_proj.weight"), need(t, "k_proj.weight"), need(t, "v_proj.weight")});
     w_o_ = need(t, "o_proj.weight");
+  }
+  // Head norms, rotation and cache store run as one launch when the norms are weighted row scales with one eps
+  // and the position encoding is a rotation by tables; any other kind runs through its own methods, step by step.
+  // Asked when the sub-parts have their tensors (a norm's weight, a rotation's tables).
+  bool fused() {
     for (Norm* n : {q_norm_.get(), k_norm_.get()})
-      if (n && !n->row_scale_weight()) throw ConfigError("attention: the native engine needs head norms that are a weighted row scale");
-    if (position_ && !position_->cos_table()) throw ConfigError("attention: the native engine needs a rotation by table");
+      if (n && !n->row_scale_weight()) return false;
+    if (q_norm_ && k_norm_ && q_norm_->eps() != k_norm_->eps()) return false;
+    return !position_ || position_->cos_table() != nullptr;
   }
   CacheNeed cache_need() const override {
     CacheNeed n;
@@ -266,11 +330,16 @@ class Attention : public Mixer {
     if (gf) ws_t = ctx.workspace(gf);
     const Tensor* ws = gf ? &ws_t : nullptr;
     const Tensor qkv = k.gemm(x, cache.writable ? w_qkv_ : w_qkv_.rows(0, (int64_t)nq_ * d_), ws);
-    const Norm* en = q_norm_ ? q_norm_.get() : k_norm_.get();
-    Tensor q = k.qkv_post(qkv, nq_, cache.writable ? nkv_ : 0, d_, &cache.k, &cache.v, cache.page_size,
-                          q_norm_ ? q_norm_->row_scale_weight() : nullptr, k_norm_ ? k_norm_->row_scale_weight() : nullptr,
-                          en ? en->eps() : 0.f, position_ ? position_->cos_table() : nullptr,
-                          position_ ? position_->sin_table() : nullptr, &ctx.positions, &tables.slots);
+    Tensor q;
+    if (fused()) {
+      const Norm* en = q_norm_ ? q_norm_.get() : k_norm_.get();
+      q = k.qkv_post(qkv, nq_, cache.writable ? nkv_ : 0, d_, &cache.k, &cache.v, cache.page_size,
+                     q_norm_ ? q_norm_->row_scale_weight() : nullptr, k_norm_ ? k_norm_->row_scale_weight() : nullptr,
+                     en ? en->eps() : 0.f, position_ ? position_->cos_table() : nullptr,
+                     position_ ? position_->sin_table() : nullptr, &ctx.positions, &tables.slots);
+    } else {
+      q = unfused(qkv, ctx, cache, tables);
+    }
     Tensor out = k.empty(q.shape);
     AttentionItems& m = items(*ctx.host);
     const Tensor& prefill_items = ctx.inputs.at("attention.prefill_items");
@@ -287,6 +356,26 @@ class Attention : public Mixer {
   }
 
  private:
+  // Norm, position encoding and store as separate steps, each sub-part through its own methods.
+  Tensor unfused(const Tensor& qkv, StepContext& ctx, CacheEntry& cache, GroupTables& tables) {
+    Kernels& k = kernels;
+    const int64_t T = qkv.dim(0), qw = (int64_t)nq_ * d_, kw = (int64_t)nkv_ * d_;
+    Tensor q = k.columns(qkv, 0, qw).view({T, nq_, d_});
+    if (q_norm_) q = q_norm_->forward(q);
+    if (!cache.writable) {
+      if (position_) q = position_->apply(q, Tensor(), ctx.positions).first;
+      return q;
+    }
+    Tensor kk = k.columns(qkv, qw, kw).view({T, nkv_, d_});
+    if (k_norm_) kk = k_norm_->forward(kk);
+    if (position_) std::tie(q, kk) = position_->apply(q, kk, ctx.positions);
+    Tensor kv = k.empty({T, 2 * kw});
+    k.copy_columns(kv, 0, kk.view({T, kw}), 0, kw);
+    k.copy_columns(kv, kw, qkv, qw + kw, kw);
+    k.qkv_post(kv, 0, nkv_, d_, &cache.k, &cache.v, cache.page_size, nullptr, nullptr, 0.f, nullptr, nullptr, nullptr, &tables.slots);
+    return q;
+  }
+
   int64_t hidden_;
   int nq_, nkv_, d_;
   float scale_;

@@ -2,7 +2,9 @@
 // and parameters as the Python package's parts (vosti_amd/parts), chosen by the same descriptions, and the
 // same kernels below them.  No part knows which model it is in.
 //
-// A new kind is one class and one register_part() call; an architecture names it in its description.
+// A new kind is one class and one register_part() call; an architecture names it in its description.  Kinds
+// and architectures can also come from outside this library: load_plugin() loads a shared library that was
+// compiled against these headers and calls its vosti_plugin_register(), which registers what it brings.
 #pragma once
 #include <functional>
 #include <map>
@@ -110,6 +112,9 @@ class PositionEncoding : public Part {
   // A rotation by tabulated angles gives its tables [positions, half]; a mixer may then rotate inside a launch of its own.
   virtual const Tensor* cos_table() { return nullptr; }
   virtual const Tensor* sin_table() { return nullptr; }
+  // Encodes positions [T] into q [T, heads, d] and k [T, kv heads, d]; k may have no memory (only q is wanted).
+  // The default rotates by the tables above; a kind without tables brings its own.
+  virtual std::pair<Tensor, Tensor> apply(const Tensor& q, const Tensor& k, const Tensor& positions);
 };
 
 class Mixer : public Part {
@@ -158,5 +163,13 @@ std::unique_ptr<T> build_part(const std::string& category, const PartSpec& spec,
 }
 
 void register_standard_parts();   // the kinds the Qwen3 dense decoder is made of
+bool part_registered(const std::string& category, const std::string& kind);
+bool block_registered(const std::string& kind);
+// Why this registry cannot build the model, or "" if it can: the first part or block kind that is missing.
+std::string missing_part(const ModelSpec& spec);
+
+// Loads a shared library and calls its `extern "C" void vosti_plugin_register(void)`, in which it registers
+// part kinds (register_part, register_block) and architectures (register_architecture).  A path is loaded once.
+void load_plugin(const std::string& path);
 
 }  // namespace vosti

@@ -104,7 +104,7 @@ class Engine:
         sampled: list[int] = []
         if sampling and self.observer.active:
             self.observer.rows(self.kernels.to_f32(logits).cpu().numpy(), [rows.index(r) for r in sampling], self.steps,
-                               str(self.kernels.dtype))
+                               str(self.kernels.dtype).replace("torch.", ""))
         if sampling:
             temps = np.zeros(len(sampling), dtype=np.float32)
             unis = np.zeros(len(sampling), dtype=np.float32)

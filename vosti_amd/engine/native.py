@@ -1,11 +1,12 @@
-"""The native engine behind the Python entry point.
+"""The engine behind the Python entry point.
 
-``NativeEngine`` has the face of ``Engine`` (``add_request``, ``step``, ``generate``, ``has_unfinished``) and
-runs plan -> forward -> sample -> commit in C++ (``csrc/engine``, built as ``libvosti_engine.so``): the same
-kernels, cache manager and scheduler, without the Python host code between two steps, which at batch 8 of
-the Qwen3-8B shape is 0.2 of a step's 4.85 ms.  It serves the parts that are built into it; models made of
-parts that are registered from Python run through ``Engine``.  For the same requests and settings both
-produce the same tokens (tests/test_native_engine_gpu.py).
+``NativeEngine`` is the engine: plan -> forward -> sample -> commit in C++ (``csrc/engine``, built as
+``libvosti_engine.so``), with the face ``add_request``, ``step``, ``generate``, ``has_unfinished``.  It serves
+every model whose architecture and part kinds are registered in the library or in a plugin loaded into it
+(``load_plugin``); ``native_support`` asks the library.  A model made of parts that exist in Python alone
+runs through ``vosti_amd.engine.Engine``, the Python step function over the same kernels, cache manager and
+scheduler; ``vosti_amd.engine.create_engine`` picks.  For the same requests and settings both produce the
+same tokens and logits (tests/test_native_engine_gpu.py).
 """
 from __future__ import annotations
 
@@ -20,7 +21,7 @@ from ..kernels import build
 from ..kernels.ops import dtype_name
 from ..sampling import SamplingParams
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 _LIB = None
 
 
@@ -32,10 +33,15 @@ def _lib():
     global _LIB
     if _LIB is None:
         import torch  # noqa: F401  (one HIP runtime per process: torch's, loaded first)
-        lib = ctypes.CDLL(str(build.ensure("engine_lib")))
+        from ..cache.host import host_lib
+        host_lib()        # linked against it: one cache manager, scheduler and registry of architectures per process
+        # Global, so that a plugin loaded later finds the registries it registers with.
+        lib = ctypes.CDLL(str(build.ensure("engine_lib")), mode=ctypes.RTLD_GLOBAL)
         lib.ve_abi_version.restype = c_int
         if lib.ve_abi_version() != ABI_VERSION:
             raise NativeEngineError(f"libvosti_engine.so has ABI {lib.ve_abi_version()}, expected {ABI_VERSION}; rebuild it")
+        lib.ve_load_plugin.argtypes = [c_char_p, c_char_p, c_int]
+        lib.ve_supports.argtypes = [c_char_p, c_char_p, c_int]
         lib.ve_create.restype = c_void_p
         lib.ve_create.argtypes = [c_char_p, c_char_p, c_char_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_uint64,
                                   c_char_p, c_int]
@@ -55,6 +61,34 @@ def _lib():
         lib.ve_trace_finish.argtypes = [c_void_p, c_int64, c_char_p, c_int]
         _LIB = lib
     return _LIB
+
+
+def load_plugin(path: str | Path) -> None:
+    """Loads a shared library that registers part kinds and architectures of its own with the native engine
+    (compiled against csrc/engine/parts.h; it exports ``vosti_plugin_register``)."""
+    err = ctypes.create_string_buffer(2048)
+    if _lib().ve_load_plugin(str(path).encode(), err, len(err)) != 0:
+        raise NativeEngineError(err.value.decode(errors="replace"))
+
+
+def load_plugins_from_environment() -> None:
+    """VOSTI_PLUGINS: paths of plugins, separated by colons, as the native program reads it."""
+    import os
+    for path in (os.environ.get("VOSTI_PLUGINS") or "").split(":"):
+        if path:
+            load_plugin(path)
+
+
+def native_support(model_dir: str | Path) -> tuple[bool, str]:
+    """Whether the native engine can run the model in ``model_dir``, and if not, why: (False, reason) when the
+    architecture or one of its part kinds is registered only in Python.  A configuration that breaks a rule
+    raises ``ConfigError`` with the library's text."""
+    from ..config import ConfigError
+    err = ctypes.create_string_buffer(2048)
+    rc = _lib().ve_supports(str(model_dir).encode(), err, len(err))
+    if rc < 0:
+        raise ConfigError(err.value.decode(errors="replace"))
+    return rc == 1, err.value.decode(errors="replace")
 
 
 class NativeEngine:

@@ -20,9 +20,11 @@ def build_parser() -> argparse.ArgumentParser:
     p.add_argument("--prefix-cache", action="store_true",
                    help="a request whose first tokens equal full pages that an earlier request left reuses those pages: "
                         "feed such a request its tokens from the first uncached one on (--prefix-report tells which)")
-    p.add_argument("--engine", default="python", choices=["python", "native"],
-                   help="which step function runs the trace: the Python one (engine/step.py) or the native engine's "
-                        "(csrc/engine/runner.cpp); the same kernels, cache manager and logits")
+    p.add_argument("--engine", default="auto", choices=["auto", "native", "python"],
+                   help="which step function runs the trace: the native engine's (csrc/engine/runner.cpp), or the Python one "
+                        "(engine/step.py) for a model whose parts exist in Python alone; auto asks the library which it is. "
+                        "The same kernels, cache manager and logits")
+    p.add_argument("--plugin", action="append", default=[], help="a shared library of parts for the native engine (may be repeated)")
     p.add_argument("--prefix-report", default=None,
                    help="a file that gets one line '<id> <cached tokens>' when a request with a 'prompt' field is first seen")
     return p
@@ -39,7 +41,18 @@ def main(argv: list[str] | None = None) -> int:
         return 2
     page = args.page_size
     num_pages = max(1, -(-args.max_tokens // page))
-    if args.engine == "native":
+    which = args.engine
+    if which != "python":
+        from .native import load_plugin, load_plugins_from_environment, native_support
+        load_plugins_from_environment()
+        for path in args.plugin:
+            load_plugin(path)
+        supported, why = native_support(args.model)
+        if which == "native" and not supported:
+            print(f"trace_run: --engine native: {why}", file=sys.stderr)
+            return 2
+        which = "native" if supported else "python"
+    if which == "native":
         from .native import NativeEngine
         native = NativeEngine(args.model, dtype=args.dtype, num_pages=num_pages, page_size=page, max_num_seqs=args.max_requests,
                               enable_prefix_cache=args.prefix_cache, graphs=False)
@@ -68,6 +81,7 @@ def main(argv: list[str] | None = None) -> int:
     out_dir = Path(args.out)
     out_dir.mkdir(parents=True, exist_ok=True)
     ids: dict[str, int] = {}     # request names -> numbers; a name may come back after it ended
+    fed: dict[str, int] = {}     # request names -> tokens the request holds so far (cached prefix included)
     next_id = 0
     print("trace_run: ready", file=sys.stderr, flush=True)
     for line in sys.stdin:
@@ -93,12 +107,23 @@ def main(argv: list[str] | None = None) -> int:
                     if skip < 0:
                         raise SystemExit(f"trace_run: request {name} starts at {e.get('start', 0)} but {cached} tokens are cached")
                     e = dict(e, tokens=e["tokens"][skip:], want=[w - skip for w in e.get("want", []) if w >= skip])
+                    fed[name] = cached
+                else:
+                    fed[name] = int(e.get("start", 0)) if "start" in e else 0
             entries.append((ids[name], [int(t) for t in e["tokens"]], [int(w) for w in e.get("want", [])]))
+        # Which row of the step's file is which: [request id, position of the token in the request] per wanted place.
+        index = []
+        for e, (rid, tokens, want) in zip(rec.get("entries", []), entries):
+            name = str(e["id"])
+            index += [[e["id"], fed.get(name, 0) + w] for w in want]
+            fed[name] = fed.get(name, 0) + len(tokens)
         logits = step_logits(entries)
         if logits.shape[0] > 0:
             logits.astype("<f4", copy=False).tofile(str(out_dir / f"{step}.f32"))
+            (out_dir / f"{step}.json").write_text(json.dumps({"step": step, "rows": index, "vocab": int(logits.shape[1])}))
         for name in rec.get("end", []):
             name = str(name)
+            fed.pop(name, None)
             if name in ids:
                 rid = ids.pop(name)
                 if has_request(rid):

@@ -6,11 +6,13 @@ Three shared libraries and one program are built from ``vosti_amd/csrc``:
   sources compiled with ``-DVK_BF16`` or ``-DVK_F32`` (hipcc);
 * ``libvosti_host.so``: the cache manager, the scheduler, the architectures' reading of config.json and
   the rules that every host of the kernels shares (g++, no GPU code);
-* ``vosti_engine``: the native engine and its command line (``csrc/engine`` with
-  the cache manager and the scheduler compiled in; g++ against the HIP runtime;
-  it loads the kernel library of the chosen precision from its own folder), and
-  ``libvosti_engine.so``: the same engine behind a C interface (``capi.cpp``
-  instead of ``main.cpp``), which ``vosti_amd.engine.NativeEngine`` drives.
+* ``libvosti_engine.so``: the native engine (``csrc/engine`` but its command
+  line; g++ against the HIP runtime, linked against ``libvosti_host.so``, so that
+  a process has one cache manager, one scheduler and one registry of
+  architectures; it loads the kernel library of the chosen precision from its own
+  folder), with a C interface (``capi.cpp``) that ``vosti_amd.engine.NativeEngine``
+  drives;
+* ``vosti_engine``: the engine's command line (``main.cpp``), linked against the two.
 
 A library is rebuilt when the hash of its sources, headers and flags differs
 from the one recorded beside it.  ``ensure()``
@@ -93,11 +95,10 @@ def _sources(name: str) -> tuple[list[Path], list[Path]]:
         return sorted(host.glob("*.cpp")), sorted(host.glob("*.h"))
     if name in ("engine", "engine_lib"):
         engine = CSRC / "engine"
-        face = "capi.cpp" if name == "engine" else "main.cpp"       # the file of the other face is left out
-        # Everything of the host library but its C interface and the plain references of the kernels.
-        shared = [p for p in sorted(host.glob("*.cpp")) if p.name not in ("capi.cpp", "reference.cpp")]
-        return ([p for p in sorted(engine.glob("*.cpp")) if p.name != face] + shared,
-                sorted(engine.glob("*.h")) + sorted(host.glob("*.h")))
+        headers = sorted(engine.glob("*.h")) + sorted(host.glob("*.h"))
+        if name == "engine":
+            return [engine / "main.cpp"], headers
+        return [p for p in sorted(engine.glob("*.cpp")) if p.name != "main.cpp"], headers
     return sorted(CSRC.glob("*.hip")), sorted(CSRC.glob("*.h"))
 
 
@@ -163,10 +164,19 @@ def build(name: str, verbose: bool = True) -> Path:
     with ThreadPoolExecutor(workers) as pool:
         objs = list(pool.map(compile_one, srcs))
     out = lib_dir() / _file_name(name)
+    # The engine's library is linked against the host library and the program against both; they find each
+    # other in their own folder at run time ($ORIGIN), or where they were when this was linked.
+    needs = {"engine_lib": ["host"], "engine": ["engine_lib", "host"]}.get(name, [])
+    deps: list[str] = []
+    for dep in needs:
+        dep_path = ensure(dep, verbose)
+        deps += ["-L", str(dep_path.parent), f"-l{dep_path.name[3:-3]}", f"-Wl,-rpath,{dep_path.parent}"]
+    if needs:
+        deps.append("-Wl,-rpath,$ORIGIN")
     if name == "engine":
         tmp = out.with_name(f"{out.name}.tmp{os.getpid()}")
         rocm_lib = str(rocm_root() / "lib")
-        _run([compiler, "-o", str(tmp), *map(str, objs), "-L", rocm_lib, "-lamdhip64", "-ldl", f"-Wl,-rpath,{rocm_lib}"], out.name)
+        _run([compiler, "-o", str(tmp), *map(str, objs), *deps, "-L", rocm_lib, "-lamdhip64", "-ldl", f"-Wl,-rpath,{rocm_lib}"], out.name)
         os.replace(tmp, out)
         Path(str(out) + ".srchash").write_text(source_hash(name) + "\n")
         if verbose:
@@ -176,7 +186,7 @@ def build(name: str, verbose: bool = True) -> Path:
     link = [compiler, "-shared", "-fPIC", "-o", str(tmp), *map(str, objs)]
     if name == "engine_lib":
         rocm_lib = str(rocm_root() / "lib")
-        link += ["-L", rocm_lib, "-lamdhip64", "-ldl", f"-Wl,-rpath,{rocm_lib}"]
+        link += [*deps, "-L", rocm_lib, "-lamdhip64", "-ldl", f"-Wl,-rpath,{rocm_lib}"]
     elif name != "host":
         link.insert(1, f"--offload-arch={GPU_ARCH}")
     _run(link, out.name)
@@ -195,7 +205,9 @@ def build(name: str, verbose: bool = True) -> Path:
 
 
 def ensure(name: str, verbose: bool = True) -> Path:
-    """Return the path of an up-to-date library, compiling it if needed."""
+    """Return the path of an up-to-date library, compiling it (and what it is linked against) if needed."""
+    for dep in {"engine_lib": ["host"], "engine": ["host", "engine_lib"]}.get(name, []):
+        ensure(dep, verbose)
     if is_current(name):
         return lib_path(name)
     if verbose:
@@ -203,8 +215,19 @@ def ensure(name: str, verbose: bool = True) -> Path:
     return build(name, verbose)
 
 
+def build_plugin(source: str | Path, out: str | Path) -> Path:
+    """Compiles one C++ file that registers part kinds or architectures with the native engine into a shared
+    library for ``load_plugin`` (host compiler; the engine's headers are csrc/engine and csrc/host).  What it
+    uses of the engine is resolved when it is loaded into a process that holds the engine."""
+    compiler = _find("g++", "/usr/bin/g++")
+    out = Path(out)
+    _run([compiler, *HOST_FLAGS, "-shared", "-I", str(CSRC / "engine"), "-I", str(CSRC / "host"), "-I", str(rocm_root() / "include"),
+          str(source), "-o", str(out)], Path(source).name)
+    return out
+
+
 def build_all(verbose: bool = True) -> None:
-    for name in ("host", "engine", "engine_lib", "bf16", "f32"):
+    for name in ("host", "engine_lib", "engine", "bf16", "f32"):
         build(name, verbose)
 
 

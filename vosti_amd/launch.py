@@ -21,6 +21,8 @@ here; each also has a command-line option, which wins:
     VOSTI_OUTPUT_TOKENS        --output-tokens       write "index<TAB>ids" lines to this file
     VOSTI_BENCH_INPUT          --bench-input         TSV of MAX_TOKENS<TAB>IDS[<TAB>ARRIVAL_STEP] requests
     VOSTI_BENCH_WARMUP_INPUT   --bench-warmup-input  a TSV of other requests, served first by the same engine
+    VOSTI_BENCH_GRAPH_PRIMER_INPUT --bench-graph-primer-input  a third TSV, served before the warm-up, so that the
+                                                     recordings of its decode steps exist before anything is timed
     VOSTI_BENCH_CALLS          --bench-calls         JSON of several calls served one after the other by one engine
     VOSTI_BENCH_CALL_RESULTS   --bench-call-results  where their records go (a new JSON file)
     VOSTI_MAX_MODEL_LEN        --max-model-len       longest prompt plus output (default: the model's positions)
@@ -31,9 +33,16 @@ here; each also has a command-line option, which wins:
 Options without a counterpart in the reference: VOSTI_DTYPE / --dtype (bfloat16,
 float32), VOSTI_TEMPERATURE / --temperature, VOSTI_SEED / --seed,
 VOSTI_PAGE_SIZE / --page-size, VOSTI_PREFIX_CACHE / --prefix-cache (0, 1),
-VOSTI_ENGINE / --engine (python, native: the same engine driven from C++,
-``vosti_amd.engine.NativeEngine``; the whole launcher as a native program is
-``bin/vosti_engine``).
+VOSTI_PLUGINS / --plugin (shared libraries that bring part kinds and
+architectures to the native engine).
+
+Who serves: the native engine's program (``vosti_amd/_lib/vosti_engine``,
+csrc/engine/main.cpp), started as a child process with these options and this
+environment, as the reference's launcher starts its engine example.  Only a model
+whose architecture or parts exist in Python alone (registered with
+``vosti_amd.config.register_architecture`` / ``vosti_amd.parts.register_part``) is
+served by the Python step function in this process; the library is asked which
+it is.  VOSTI_ENGINE / --engine (auto, native, python) overrides that, for tests.
 End tokens come from generation_config.json's ``eos_token_id`` (one to three
 ids: python/vosti_kernels/serving_workload.py:78-108); without that file there
 are none.  It prints ``MODEL_OUTPUT_TOKEN_IDS=[...]`` like the reference, or a
@@ -51,9 +60,30 @@ from pathlib import Path
 
 
 def families() -> dict[str, str]:
-    """--family names: the ``model_type`` of every registered architecture -> its name."""
+    """--family names: the ``model_type`` of every registered architecture -> its name (those of the native
+    library and its plugins, and those registered in Python)."""
     from .config.registry import model_types
+    if os.environ.get("VOSTI_PLUGINS"):
+        from .engine.native import load_plugins_from_environment
+        load_plugins_from_environment()
     return model_types()
+
+
+def run_native_program(argv: list[str], family: str, dtype: str) -> int:
+    """The native engine's program with the launcher's options and environment, as a child process."""
+    import subprocess
+    from .kernels import build
+    program = build.ensure("engine")
+    lib = build.ensure({"bfloat16": "bf16", "float32": "f32"}[dtype])
+    args, skip = [], False
+    for a in argv:                       # --engine is this launcher's own
+        if skip:
+            skip = False
+        elif a == "--engine":
+            skip = True
+        elif not a.startswith("--engine="):
+            args.append(a)
+    return subprocess.run([str(program), "--family", family, *args, "--lib-dir", str(lib.parent)]).returncode
 
 
 def _env(name: str, default=None):
@@ -84,7 +114,9 @@ def engine_parser() -> argparse.ArgumentParser:
     p.add_argument("--seed", type=int, default=int(_env("VOSTI_SEED", 0)))
     p.add_argument("--page-size", type=int, default=int(_env("VOSTI_PAGE_SIZE", 64)))
     p.add_argument("--prefix-cache", type=int, default=int(_env("VOSTI_PREFIX_CACHE", 1)), choices=[0, 1])
-    p.add_argument("--engine", default=_env("VOSTI_ENGINE", "python"), choices=["python", "native"])
+    p.add_argument("--bench-graph-primer-input", default=_env("VOSTI_BENCH_GRAPH_PRIMER_INPUT"))
+    p.add_argument("--plugin", action="append", default=[], help="a shared library of parts for the native engine (may be repeated)")
+    p.add_argument("--engine", default=_env("VOSTI_ENGINE", "auto"), choices=["auto", "native", "python"])
     return p
 
 
@@ -194,6 +226,17 @@ def run_engine(argv: list[str], family: str) -> int:
         raise SystemExit("MODEL_PATH (or --model-path) is required")
     if args.device not in ("cuda:0", "cuda"):
         raise SystemExit(f"device {args.device!r}: this engine runs on cuda:0 only")
+    which = args.engine
+    if which != "python":
+        from .engine.native import load_plugin, native_support
+        for path in args.plugin:
+            load_plugin(path)
+        supported, why = native_support(args.model_path)
+        if which == "native" and not supported:
+            raise SystemExit(f"--engine native: {why}")
+        which = "native" if supported else "python"
+    if which == "native":
+        return run_native_program(argv, family, args.dtype)
     from .config import load_config
     cfg = load_config(args.model_path)
     if cfg.architecture != families()[family]:
@@ -207,13 +250,10 @@ def run_engine(argv: list[str], family: str) -> int:
     else:
         requests = [(args.max_tokens, parse_ids(args.prompt_ids), 0)]
     warmup = parse_prepared(args.bench_warmup_input) if args.bench_input and args.bench_warmup_input else []
+    primer = parse_prepared(args.bench_graph_primer_input) if warmup and args.bench_graph_primer_input else []
     eos = eos_ids(args.model_path)
-    if args.engine == "native":
-        if args.bench_calls or os.environ.get("VOSTI_LOGITS_DIGEST") or os.environ.get("VOSTI_LOGITS_OBSERVER_DIR"):
-            raise SystemExit("--engine native serves neither the multi-call driver nor the logits observers; use --engine python")
-        from .engine import NativeEngine as Engine
     engine = Engine(args.model_path, dtype=args.dtype, num_pages=args.num_blocks, page_size=args.page_size,
-                    max_num_seqs=args.max_seqs or max(len(requests), len(warmup), 1 if not args.bench_calls else 8),
+                    max_num_seqs=args.max_seqs or max(len(requests), len(warmup), len(primer), 1 if not args.bench_calls else 8),
                     max_num_batched_tokens=args.max_batched_tokens, enable_prefix_cache=bool(args.prefix_cache),
                     max_model_len=args.max_model_len or None, graphs=bool(args.graphs))
     if args.bench_calls:
@@ -222,9 +262,6 @@ def run_engine(argv: list[str], family: str) -> int:
     import torch
 
     def cache_counters():
-        if args.engine == "native":
-            st = engine.stats()
-            return st["prefix_hit_requests"], st["prefix_hits"]
         return engine.cache.prefix_hit_requests(), engine.cache.prefix_hits()
 
     def serve(reqs, first_seed):
@@ -246,12 +283,20 @@ def run_engine(argv: list[str], family: str) -> int:
         text = f"{tag} batch={len(reqs)} prompt_tokens={sum(len(i) for _, i, _ in reqs)} output_tokens={n_out} wall_s={wall:.9f}"
         return text + (f" tok_s={n_out / wall:.6f}" if rate else "")
 
+    if primer:
+        # An optional third workload, served first in the same engine, so that the captures of the decode steps it
+        # walks through exist before the warm-up (examples/support/engine_serving.rs:162-181); nothing is reported of it.
+        os.environ["VOSTI_LOGITS_OBSERVER_PHASE"] = "primer"
+        serve(primer, args.seed + len(requests) + len(warmup))
     if warmup:
         # The reference serves a disjoint warm-up workload in the same engine before the measured one
         # (examples/support/engine_serving.rs:157-206) and reports both (engine_benchmark.rs:45-76).
+        os.environ["VOSTI_LOGITS_OBSERVER_PHASE"] = "warmup"
         w_out, w_wall, w_stats = serve(warmup, args.seed + len(requests))
         print(line("WARMUP", warmup, w_out, w_wall, rate=False))
         print("WARMUP_CACHE_STATS " + json.dumps(w_stats, separators=(",", ":")))
+    if warmup:
+        os.environ["VOSTI_LOGITS_OBSERVER_PHASE"] = "measured"
     outputs, wall, stats = serve(requests, args.seed)
     if trace:
         trace.close()
@@ -259,13 +304,12 @@ def run_engine(argv: list[str], family: str) -> int:
         Path(args.output_tokens).write_text("".join(f"{i}\t{','.join(map(str, o))}\n" for i, o in enumerate(outputs)))
     if args.bench_input:
         print(line("BENCH", requests, outputs, wall, rate=True))
-        stats["preemptions"] = engine.stats()["preemptions"] if args.engine == "native" else engine.scheduler.preemptions()
+        stats["preemptions"] = engine.scheduler.preemptions()
         print("CACHE_STATS " + json.dumps(stats, separators=(",", ":")))
     else:
         print(f"MODEL_OUTPUT_TOKEN_IDS={outputs[0]}")
     if args.graphs:
-        graph_stats = engine.stats()["graph_stats"] if args.engine == "native" else engine.runner.graph_stats
-        print("GRAPH_STATS " + json.dumps(graph_stats, separators=(",", ":")))
+        print("GRAPH_STATS " + json.dumps(engine.runner.graph_stats, separators=(",", ":")))
     return 0
 
 
