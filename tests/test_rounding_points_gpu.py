@@ -51,10 +51,10 @@ def head_norm_rope_variant(x, w, eps, cos, sin, positions, how):
     return bf(torch.cat([x1 * c - x2 * s, x2 * c + x1 * s, n[..., 2 * half:]], dim=-1))
 
 
-@pytest.mark.parametrize("T,H", [(24, 4096), (40, 96), (30, 100), (6, 16384), (3, 40000)])
+@pytest.mark.parametrize("T,H", [(24, 4096), (40, 96), (30, 100), (6, 16384), (3, 32768)])
 def test_add_norm_sees_the_unrounded_sum(T, H):
     """Rows in registers (4,096), short rows, a width that no vector divides (100), rows kept in LDS (16,384 and
-    40,000).  The residual is three eighths of a step of x, up or down, so that the sum is exact in 32-bit and
+    32,768).  The residual is three eighths of a step of x, up or down, so that the sum is exact in 32-bit and
     its rounding always loses that much: the two variants then differ in more than a third of the outputs
     (with a random residual in a fifth)."""
     k = kern(BF)
