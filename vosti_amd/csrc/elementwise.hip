@@ -350,8 +350,9 @@ int vk_rope_tables(elem_t* cos_t, elem_t* sin_t, const float* inv_freq, int max_
   return vk_check_launch("rope_tables");
 }
 
-// Reads `bytes` bytes at p (16-byte aligned) once and keeps nothing; `sink`: four bytes of device memory that are
-// practically never written.  For measurements only.
+// The measurements' yardstick, no part of any model: reads `bytes` bytes at p (16-byte aligned) once and keeps
+// nothing, so that a projection's time can be set against what a plain read of its weights takes on the same
+// machine (bench.py's read_only_us).  `sink`: four bytes of device memory that are practically never written.
 int vk_pull(const void* p, int64_t bytes, void* sink, hipStream_t st) {
   VK_REQUIRE(p != nullptr && sink != nullptr && ((uintptr_t)p % 16) == 0 && bytes >= 16, "pull: bad operands");
   const int64_t n16 = bytes / 16;

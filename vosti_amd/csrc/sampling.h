@@ -19,8 +19,7 @@ int vk_sample(int32_t* out, const elem_t* logits, const float* temps, const floa
 
 // vk_sample without the scratch argument, for callers that cannot allocate device memory: code under
 // HIP graph capture, tight serving loops, harnesses that forbid it.  It has no counterpart in the
-// reference, whose sampler is a library argmax (python/vosti_kernels/kernels.py:1079-1104).  The
-// partial results live in an array of the library's own, VK_SAMPLE_STATIC_MAX_ROWS * 256 bytes per GPU
+// reference.  The partial results live in an array of the library's own, VK_SAMPLE_STATIC_MAX_ROWS * 256 bytes per GPU
 // (256 KB), held from the first call on that GPU until the process ends; the call allocates and frees
 // nothing.  More rows than VK_SAMPLE_STATIC_MAX_ROWS are refused with an error.  Every call on a GPU
 // uses that GPU's one array: calls that overlap on one GPU (two streams, two host threads) race and
