@@ -396,9 +396,10 @@ def test_attention_prompt_kernels_agree(dtype, nq, nkv, d, P, window):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_attention_many_decoded_tokens(dtype):
-    """The decode kernels: keys split over workgroups by segment, with few workgroups (keys and values
-    asked for together) and with more than a thousand (values later), and one workgroup per token and
-    kv head: the plain result and the same bits, with and without a window, for groups of 1 and 20 q heads."""
+    """The decode kernels: a wave per segment that asks for a tile's fragments when it needs them, with few waves
+    (keys and values asked for together) and with more than a thousand (values later), a wave per segment with the
+    next tile's fragments in flight, and two waves per segment: the plain result and the same bits, with and
+    without a window, for groups of 1 and 20 q heads."""
     k = kern(dtype)
     P = 16
     for nq, nkv, d, window in ((8, 8, 64, 0), (8, 8, 64, 300), (20, 1, 48, 0)):
@@ -423,9 +424,9 @@ def test_attention_many_decoded_tokens(dtype):
                                                (4, 2, 80, 64, 130)])
 def test_attention_decode_kernels_agree(dtype, nq, nkv, d, P, window):
     """Decoded tokens after contexts that end at every place of a tile, a segment and a page, through
-    the kernel with a wave per tile, the one with a wave per segment and the one with two waves per
-    segment (head sizes and pages they know at compile time, and one they do not): the same bits, and the
-    plain result."""
+    the kernel that asks for a tile's fragments when it needs them, the one with the next tile's fragments
+    in flight and the one with two waves per segment (head sizes and pages they know at compile time, and one
+    they do not): the same bits, and the plain result."""
     k = kern(dtype)
     lens = [1, 2, 63, 64, 65, 255, 256, 257, 320, 511, 512, 513, 1023, 1024, 1025, 1300, 1793, 2047, 2048, 2049]
     q_list = [rand((1, nq, d), dtype, 10 + i) for i in range(len(lens))]

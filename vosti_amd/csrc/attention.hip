@@ -13,26 +13,29 @@
 // Reduction order.  It is a function of absolute key positions only, so that
 // any cut of a sequence into steps, and any split of the keys over waves and
 // workgroups, gives the same bits:
-//   tile     64 keys, positions 64t .. 64t+63.  Each tile is reduced on its
-//            own: m = (max of the visible raw scores) * c with c = scale * log2(e),
-//            p = 2^(fma(raw, c, -m)), l = sum p, acc = P V accumulated from zero.
-//            A tile without a visible key is empty (m = -inf).
-//   segment  4 tiles (256 keys).  Its non-empty tiles are folded, ascending,
-//            into a state that starts empty:
+//   tile     64 keys, positions 64t .. 64t+63.
+//   segment  4 tiles (256 keys).  A row's state (M, L, ACC) of a segment starts empty (M = -inf) and takes
+//            in the segment's tiles in ascending order, each as the reference's kernel takes in a block of
+//            keys (fattn_paged.py:198-262): with c = scale * log2(e) and m = (max of the tile's visible raw
+//            scores) * c,
+//              M' = m if the state is empty or m > M + 8, else M (the reference point moves only when the
+//              maximum grows by more than 2^8: a probability is then at most 2^8, and the sums so far are
+//              scaled in few tiles instead of in most); a = 2^(M - M');
+//              p = 2^(fma(raw, c, -M')) (0 for a key the row does not see);
+//              L' = fma(L, a, sum p); ACC' = ACC * a + P V, the product accumulated onto ACC * a by the
+//            matrix unit, key slab after key slab.  A tile in which the row sees no key changes nothing.
+//   total    the non-empty segments are folded, ascending, into a state that starts empty:
 //              M' = max(M, m); ACC' = fma(acc, 2^(m - M'), ACC * 2^(M - M')); L' likewise.
-//   total    the non-empty segments are folded, ascending, the same way.
 // Kernels, all with the same sequence of fp32 operations per row:
 //   attn_prefill_lds   prompt rows, head sizes 64/128/256 and pages of a tile or more: key and value
-//                      tiles pass through LDS once per workgroup; folds in registers.
+//                      tiles pass through LDS once per workgroup; segments and total in registers.
 //   attn_prefill       prompt rows of every shape: fragments straight from global memory.
 //   attn_decode_seg    decoded tokens: a wave walks the tiles of a segment with the next tile's
-//                      fragments in flight and folds in registers; the segment's (m, l, acc) goes
-//                      to a scratch buffer ...
+//                      fragments in flight; the segment's (M, L, ACC) goes to a scratch buffer ...
 //   attn_combine       ... which this one folds.
-//   attn_decode        the same with a wave per tile and the fold in LDS: for head and element
-//                      sizes whose fragments of two tiles do not fit a wave's registers.
-//   attn_decode_whole  decoded tokens of large batches, those sizes: all tiles of a token and kv
-//                      head in one workgroup, folded from LDS; no scratch.
+//   attn_decode_pair   the same with two waves a segment, for steps with few segments.
+//   attn_decode_plain  the same with a tile's fragments asked for when they are needed: for head and
+//                      element sizes whose fragments of two tiles do not fit a wave's registers.
 //
 // Cache layout: keys [pages, nkv, page, d]; values transposed [pages, nkv, d, page],
 // so that both MFMA operands of both products are 16-byte loads from global
@@ -49,6 +52,7 @@
 #define KEY_SLABS (TILE_KEYS / VK_SLAB)   // key slabs per tile: 2 (bfloat16) or 4 (float)
 #define S_PER_LANE 16                     // scores per lane per tile
 #define ITEM_ROWS 128                     // rows of a prompt item
+#define MAX_STEP 8.0f                     // a row's reference maximum moves when the tile's exceeds it by more than this (log2)
 
 struct AttnArgs {
   const elem_t* q;        // [T, nq, d]
@@ -80,27 +84,32 @@ struct RowCtx {
   float scale_log2;
 };
 
-// Scores of one tile -> the tile's own statistics (m, l) of this lane's row and its probabilities,
-// rounded to the element type, as MFMA operands.  The row sees keys lo..pos.  m is the largest
-// visible score times scale_log2 (> 0), a probability is 2^(score * scale_log2 - m) with the product
-// and the difference rounded once (a fused multiply-add).  `full` (the same for the whole wave) says
-// that every row of the wave sees every key of the tile: then the masks are left out, which changes
-// no bit.
-__device__ __forceinline__ void tile_softmax(float (&sc)[S_PER_LANE], int kb, int g, bool row_ok, int lo, int pos,
-                                             float scale_log2, bool full, float& m_t, float& l_t,
-                                             frag_t (&pf)[KEY_SLABS]) {
+// Scores of one tile onto the running state (M, L) of this lane's row in its segment: the new reference
+// maximum (see the top of this file), the factor `ca` that the row's sums so far have to be scaled by (ACC is the
+// caller's), L, and the tile's probabilities relative to the new maximum, rounded to the element type, as MFMA
+// operands.  The row sees keys
+// lo..pos.  A probability is 2^(score * scale_log2 - M') with the product and the difference rounded once (a fused
+// multiply-add).  `full` (the same for the whole wave) says that every row of the wave sees every key of the
+// tile: then the masks are left out, which changes no bit.  A row that sees no key of the tile keeps its state
+// (ca = 1, probabilities 0).
+__device__ __forceinline__ void tile_probs(float (&sc)[S_PER_LANE], int kb, int g, bool row_ok, int lo, int pos,
+                                           float scale_log2, bool full, float& M, float& L, float& ca,
+                                           frag_t (&pf)[KEY_SLABS]) {
   float pr[S_PER_LANE];
   float psum = 0.f;
+  float Mn;
   if (full) {
     float tmax = sc[0];
 #pragma unroll
     for (int i = 1; i < S_PER_LANE; ++i) tmax = fmaxf(tmax, sc[i]);
     tmax = fmaxf(tmax, lane_xor16(tmax));
     tmax = fmaxf(tmax, lane_xor32(tmax));
-    m_t = tmax * scale_log2;
+    const float m = tmax * scale_log2;
+    Mn = (!(M > -INFINITY) || m > M + MAX_STEP) ? m : M;
+    ca = fast_exp2(M - Mn);                 // 1 where the maximum stands, 0 for a row whose state was empty
 #pragma unroll
     for (int i = 0; i < S_PER_LANE; ++i) {
-      pr[i] = fast_exp2(__builtin_fmaf(sc[i], scale_log2, -m_t));
+      pr[i] = fast_exp2(__builtin_fmaf(sc[i], scale_log2, -Mn));
       psum = psum + pr[i];
     }
   } else {
@@ -114,16 +123,19 @@ __device__ __forceinline__ void tile_softmax(float (&sc)[S_PER_LANE], int kb, in
     }
     tmax = fmaxf(tmax, lane_xor16(tmax));
     tmax = fmaxf(tmax, lane_xor32(tmax));
-    m_t = tmax * scale_log2;
+    const float m = tmax * scale_log2;      // -inf: the row sees no key of the tile
+    Mn = (!(M > -INFINITY) || m > M + MAX_STEP) ? m : M;
+    ca = Mn > -INFINITY ? fast_exp2(M - Mn) : 1.f;
 #pragma unroll
     for (int i = 0; i < S_PER_LANE; ++i) {
-      pr[i] = vis[i] ? fast_exp2(__builtin_fmaf(sc[i], scale_log2, -m_t)) : 0.f;
+      pr[i] = vis[i] ? fast_exp2(__builtin_fmaf(sc[i], scale_log2, -Mn)) : 0.f;
       psum = psum + pr[i];
     }
   }
   psum = psum + lane_xor16(psum);
   psum = psum + lane_xor32(psum);
-  l_t = psum;
+  L = __builtin_fmaf(L, ca, psum);
+  M = Mn;
 #pragma unroll
   for (int ks = 0; ks < KEY_SLABS; ++ks) {
 #ifdef VK_BF16
@@ -132,6 +144,21 @@ __device__ __forceinline__ void tile_softmax(float (&sc)[S_PER_LANE], int kb, in
 #else
     pf[ks] = f32x4{pr[ks * 4 + 0], pr[ks * 4 + 1], pr[ks * 4 + 2], pr[ks * 4 + 3]};
 #endif
+  }
+}
+
+// ACC * ca, a row's sums so far under its new maximum.  Left out for the wave as a whole when it changes nothing:
+// every row's factor is 1 (the maximum stood), or the row's state was empty before this tile (`fresh`: its sums
+// are zero).
+template <int NDT>
+__device__ __forceinline__ void scale_state(f32x4 (&ACC)[NDT], float ca, bool fresh) {
+  if (__all(ca == 1.f || fresh)) return;
+#pragma unroll
+  for (int dt = 0; dt < NDT; ++dt) {
+    ACC[dt].x = ACC[dt].x * ca;
+    ACC[dt].y = ACC[dt].y * ca;
+    ACC[dt].z = ACC[dt].z * ca;
+    ACC[dt].w = ACC[dt].w * ca;
   }
 }
 
@@ -225,10 +252,10 @@ __device__ __forceinline__ void tile_scores(const RowCtx& c, const frag_t (&kf)[
   }
 }
 
-// acc = V^T P^T from zero; values of keys the sequence does not own count as zero.
+// ACC += V^T P^T; values of keys the sequence does not own count as zero.
 template <int NDT, bool EXACT>
 __device__ __forceinline__ void tile_pv(const RowCtx& c, int kb, frag_t (&vf)[NDT][KEY_SLABS], const frag_t (&pf)[KEY_SLABS],
-                                        f32x4 (&acc)[NDT]) {
+                                        f32x4 (&ACC)[NDT]) {
   const int d = EXACT ? NDT * 16 : c.d;
   if (kb + TILE_KEYS > c.k_len || kb < c.wave_lo) {
 #pragma unroll
@@ -237,18 +264,17 @@ __device__ __forceinline__ void tile_pv(const RowCtx& c, int kb, frag_t (&vf)[ND
   }
 #pragma unroll
   for (int dt = 0; dt < NDT; ++dt) {
-    acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
     if (dt * 16 < d) {
 #pragma unroll
-      for (int ks = 0; ks < KEY_SLABS; ++ks) acc[dt] = mma_slab(vf[dt][ks], pf[ks], acc[dt]);
+      for (int ks = 0; ks < KEY_SLABS; ++ks) ACC[dt] = mma_slab(vf[dt][ks], pf[ks], ACC[dt]);
     }
   }
 }
 
-// One tile, reduced on its own: m, l and acc[NDT] of this lane's row.
+// One tile onto the segment's state (M, L, ACC) of this lane's row, fragments straight from global memory.
 template <int NDT, int NQS, bool V_LATE, bool EXACT = false>
-__device__ __forceinline__ void tile_partial(const RowCtx& c, const frag_t (&qf)[NQS], int kb, float& m_t, float& l_t,
-                                             f32x4 (&acc)[NDT]) {
+__device__ __forceinline__ void tile_step(const RowCtx& c, const frag_t (&qf)[NQS], int kb, float& M, float& L,
+                                          f32x4 (&ACC)[NDT]) {
   frag_t kf[KSUB][NQS];
   frag_t vf[NDT][KEY_SLABS];
   load_keys<NQS, EXACT>(c, kb, kf);
@@ -263,11 +289,14 @@ __device__ __forceinline__ void tile_partial(const RowCtx& c, const frag_t (&qf)
     load_values<NDT, EXACT>(c, kb, vf);
   }
   frag_t pf[KEY_SLABS];
-  tile_softmax(sc, kb, c.g, c.row_ok, c.lo, c.pos, c.scale_log2, false, m_t, l_t, pf);
-  tile_pv<NDT, EXACT>(c, kb, vf, pf, acc);
+  float ca;
+  const bool fresh = !(M > -INFINITY);
+  tile_probs(sc, kb, c.g, c.row_ok, c.lo, c.pos, c.scale_log2, false, M, L, ca, pf);
+  scale_state<NDT>(ACC, ca, fresh);
+  tile_pv<NDT, EXACT>(c, kb, vf, pf, ACC);
 }
 
-// state (M, L, ACC) <- fold of a non-empty partial (m, l, acc).
+// state (M, L, ACC) <- fold of a non-empty segment (m, l, acc).
 __device__ __forceinline__ void fold_scales(float M, float m, float& Mn, float& ca, float& cb) {
   Mn = fmaxf(M, m);
   ca = fast_exp2(M - Mn);
@@ -361,12 +390,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a, int heads
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt) As[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
     const int t_end = min(tile_hi, seg * SEG_TILES + SEG_TILES - 1);
-    for (int t = max(tile_lo, seg * SEG_TILES); t <= t_end; ++t) {
-      float m_t, l_t;
-      f32x4 acc[NDT];
-      tile_partial<NDT, NQS, true>(c, qf, t * TILE_KEYS, m_t, l_t, acc);
-      fold<NDT>(Ms, Ls, As, m_t, l_t, acc);
-    }
+    for (int t = max(tile_lo, seg * SEG_TILES); t <= t_end; ++t) tile_step<NDT, NQS, true>(c, qf, t * TILE_KEYS, Ms, Ls, As);
     fold<NDT>(M, L, ACC, Ms, Ls, As);
   }
   if (c.row_ok) {
@@ -385,12 +409,17 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a, int heads
 }
 
 // Prompt portions, the fast kernel: head sizes 64, 128, 256 with pages of at
-// least a tile.  A workgroup is one q head and one item; each of its waves has
-// QT 16-row tiles of the item's rows.  Every key tile goes from global memory
+// least a tile.  A workgroup is one q head and one item; each of its NW waves has
+// one 16-row tile of the item's rows.  Every key tile goes from global memory
 // straight into LDS once (global_load_lds_dwordx4, two buffers: the next tile
-// lands while this one is used) and is read from there by all waves; a key or
-// value fragment read from LDS serves both row tiles of a wave.  The
-// arithmetic per row is tile_partial's and fold's, operation for operation.
+// lands while this one is used) and is read from there by all waves.  A tile's
+// work is three stretches of code that the compiler does not mix: the scores
+// (key fragments from LDS, MFMAs), the probabilities and the scaling of the
+// row's sums (vector instructions), the product with the values (value fragments
+// from LDS, MFMAs); a wave runs the two with MFMAs at a raised priority, so that
+// of the two waves of a SIMD the one that feeds the matrix unit goes first and the
+// other's vector instructions fill in.  The arithmetic per row is tile_step's and
+// fold's, operation for operation.
 //
 // LDS holds the key tile as [64 keys][d] and the value tile as [d][64 keys],
 // in 16-byte columns that are XOR-swizzled by row so that the 16 lanes of a
@@ -413,9 +442,9 @@ __device__ __forceinline__ int key_swz(int row) { return row & 15; }
 __device__ __forceinline__ int val_swz(int row) { return row & 15; }          // rows of 256 bytes
 #endif
 
-template <int DPAD, int QT, int NW>
+template <int DPAD, int NW>
 __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_lds_kernel(AttnArgs a, int n_items) {
-  constexpr int ROWS_WG = 16 * QT * NW;                  // NW waves, each with QT 16-row tiles
+  constexpr int ROWS_WG = 16 * NW;                       // NW waves, each with one 16-row tile
   constexpr int BPI = ITEM_ROWS / ROWS_WG;               // workgroups per item
   static_assert(ITEM_ROWS % ROWS_WG == 0, "a workgroup's rows must divide an item");
   constexpr int NDT = DPAD / 16, NQS = DPAD / VK_SLAB;
@@ -452,7 +481,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_lds_kernel(AttnArgs a
   const int kvh = head / (a.nq / a.nkv);
   const int seq = a.items[2 * item], q_off0 = a.items[2 * item + 1] + (block % BPI) * ROWS_WG;
   const int q_begin = a.cu_q[seq], q_len = a.cu_q[seq + 1] - q_begin;
-  if (q_off0 >= q_len) return;                           // the item ends before this workgroup's rows
+  if (q_off0 >= q_len) return;                           // the item ends before this workgroup's rows: the whole workgroup
   const int k_len = a.k_len[seq];
   const int rows_item = min(ROWS_WG, q_len - q_off0);    // this workgroup's rows
   const int pos_item = k_len - q_len + q_off0;           // position of the item's first row
@@ -460,21 +489,16 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_lds_kernel(AttnArgs a
   const int tile_lo = item_lo / TILE_KEYS, tile_hi = (pos_item + rows_item - 1) / TILE_KEYS;
 
   // ---- this wave's rows ----
-  const int rows_wave = min(16 * QT, rows_item - 16 * QT * wave);  // <= 0: the wave only helps to load
-  const int pos_wave = pos_item + 16 * QT * wave;
+  const int rows_wave = min(16, rows_item - 16 * wave);  // <= 0: the wave only helps to load
+  const int pos_wave = pos_item + 16 * wave;
   const int wave_lo = a.window > 0 ? max(0, pos_wave - a.window + 1) : 0;
   const int wtile_lo = wave_lo / TILE_KEYS, wtile_hi = rows_wave > 0 ? (pos_wave + rows_wave - 1) / TILE_KEYS : -1;
-  bool row_ok[QT];
-  int pos[QT], lo[QT], tok[QT];
-  frag_t qf[QT][NQS];
-#pragma unroll
-  for (int qt = 0; qt < QT; ++qt) {
-    row_ok[qt] = 16 * qt + r16 < rows_wave;
-    pos[qt] = pos_wave + 16 * qt + r16;
-    lo[qt] = a.window > 0 ? max(0, pos[qt] - a.window + 1) : 0;
-    tok[qt] = q_begin + q_off0 + 16 * QT * wave + 16 * qt + r16;
-    load_q<NQS>(a, tok[qt], head, row_ok[qt], g, qf[qt]);
-  }
+  const bool row_ok = r16 < rows_wave;
+  const int pos = pos_wave + r16;
+  const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+  const int tok = q_begin + q_off0 + 16 * wave + r16;
+  frag_t qf[NQS];
+  load_q<NQS>(a, tok, head, row_ok, g, qf);
 
   // ---- what this lane fetches of every tile ----
   const int64_t page_elems = (int64_t)a.P * a.d;
@@ -496,7 +520,8 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_lds_kernel(AttnArgs a
   }
   auto issue = [&](int t, int stage) {
     const int kb = t * TILE_KEYS;
-    const int64_t page = (int64_t)bt[kb >> lp] * page_stride;
+    // The page number is the same for the wave: as a scalar, its arithmetic stays off the vector unit.
+    const int64_t page = (int64_t)__builtin_amdgcn_readfirstlane(bt[kb >> lp]) * page_stride;
     const int in_page = kb & (a.P - 1);
     const elem_t* kt = kbase + page + (int64_t)in_page * DPAD;
     const elem_t* vt = vbase + page + in_page;
@@ -508,15 +533,10 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_lds_kernel(AttnArgs a
     }
   };
 
-  float M[QT], L[QT], Ms[QT], Ls[QT];
-  f32x4 ACC[QT][NDT], As[QT][NDT];
+  float M = -INFINITY, L = 0.f, Ms = -INFINITY, Ls = 0.f;
+  f32x4 ACC[NDT], As[NDT];
 #pragma unroll
-  for (int qt = 0; qt < QT; ++qt) {
-    M[qt] = Ms[qt] = -INFINITY;
-    L[qt] = Ls[qt] = 0.f;
-#pragma unroll
-    for (int dt = 0; dt < NDT; ++dt) ACC[qt][dt] = As[qt][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  }
+  for (int dt = 0; dt < NDT; ++dt) ACC[dt] = As[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   issue(tile_lo, 0);
   for (int t = tile_lo; t <= tile_hi; ++t) {
@@ -524,12 +544,28 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_lds_kernel(AttnArgs a
     wait_vm_loads();
     __syncthreads();      // tile t is in LDS; every wave is done with the other buffer
     if (t < tile_hi) issue(t + 1, stage ^ 1);
+    if (t * TILE_KEYS + TILE_KEYS > k_len || t * TILE_KEYS < item_lo) {
+      // Keys outside [item_lo, k_len) may lie in pages this sequence does not own: their values are replaced by
+      // zero in LDS, so that stale NaN or Inf cannot reach a sum (their probabilities are zero).  The first and
+      // the last tile of an item at most; the same for every wave, which all pass the second barrier.
+      const int kb = t * TILE_KEYS;
+      unsigned char* vt = lds + stage * STAGE + KT_BYTES;
+      for (int e = threadIdx.x; e < DPAD * TILE_KEYS; e += 64 * NW) {
+        const int vrow = e / TILE_KEYS, key = e % TILE_KEYS;
+        if (kb + key >= k_len || kb + key < item_lo) {
+          const int col = (key / VK_VEC) ^ val_swz(vrow);
+          *reinterpret_cast<elem_t*>(vt + vrow * VRB + col * 16 + (key % VK_VEC) * EB) = (elem_t)0.f;
+        }
+      }
+      __syncthreads();
+    }
     if (t >= wtile_lo && t <= wtile_hi) {
       const int kb = t * TILE_KEYS;
       const unsigned char* kl = lds + stage * STAGE;
       const unsigned char* vl = kl + KT_BYTES;
-      // ---- scores of both row tiles ----
-      float sc[QT][S_PER_LANE];
+      // ---- scores ----
+      float sc[S_PER_LANE];
+      __builtin_amdgcn_s_setprio(1);
 #pragma unroll
       for (int sub = 0; sub < S_PER_LANE / 4; ++sub) {
         const int krow = key_row_of(sub, r16);
@@ -538,175 +574,112 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_lds_kernel(AttnArgs a
         frag_t kf[NQS];
 #pragma unroll
         for (int s = 0; s < NQS; ++s) kf[s] = *reinterpret_cast<const frag_t*>(kr + (((s * 4 + g) ^ sw) << 4));
+        f32x4 s4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int qt = 0; qt < QT; ++qt) {
-          f32x4 s4 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-          for (int s = 0; s < NQS; ++s) s4 = mma_slab(kf[s], qf[qt][s], s4);
-          sc[qt][4 * sub + 0] = s4.x;
-          sc[qt][4 * sub + 1] = s4.y;
-          sc[qt][4 * sub + 2] = s4.z;
-          sc[qt][4 * sub + 3] = s4.w;
-        }
+        for (int s = 0; s < NQS; ++s) s4 = mma_slab(kf[s], qf[s], s4);
+        sc[4 * sub + 0] = s4.x;
+        sc[4 * sub + 1] = s4.y;
+        sc[4 * sub + 2] = s4.z;
+        sc[4 * sub + 3] = s4.w;
       }
-      // ---- each row's own statistics of this tile, and how they fold into the segment's ----
-      frag_t pf[QT][KEY_SLABS];
-      float ca[QT], cb[QT];
-      bool some[QT], all_some[QT];
-#pragma unroll
-      for (int qt = 0; qt < QT; ++qt) {
-        const bool full = rows_wave >= 16 * qt + 16 && kb + TILE_KEYS - 1 <= pos_wave + 16 * qt &&
-                          kb >= (a.window > 0 ? max(0, pos_wave + 16 * qt + 15 - a.window + 1) : 0);
-        float m_t, l_t, Mn;
-        tile_softmax(sc[qt], kb, g, row_ok[qt], lo[qt], pos[qt], a.scale_log2, full, m_t, l_t, pf[qt]);
-        some[qt] = m_t > -INFINITY;
-        all_some[qt] = __all(some[qt]);
-        fold_scales(Ms[qt], m_t, Mn, ca[qt], cb[qt]);
-        if (some[qt]) {
-          Ls[qt] = fold1(Ls[qt], l_t, ca[qt], cb[qt]);
-          Ms[qt] = Mn;
-        }
-      }
-      // ---- P V from zero, folded into the segment's sum column block by column block: fold()'s
-      // arithmetic.  When every row of the wave has a key in the tile, which is the rule, the loop
-      // has no branch and no select inside, so that the reads from LDS, the MFMAs and the folds of
-      // different column blocks overlap.
-      const bool edge = kb + TILE_KEYS > k_len || kb < wave_lo;
-      auto pv = [&](auto plain_tag, int qt) {
-        constexpr bool PLAIN = decltype(plain_tag)::value;
-#pragma unroll
-        for (int dt = 0; dt < NDT; ++dt) {
-          const int vrow = dt * 16 + r16;
-          const unsigned char* vr = vl + vrow * VRB;
-          const int sw = val_swz(vrow);
-          frag_t vf[KEY_SLABS];
-#pragma unroll
-          for (int ks = 0; ks < KEY_SLABS; ++ks) vf[ks] = *reinterpret_cast<const frag_t*>(vr + (((ks * 4 + g) ^ sw) << 4));
-          if (!PLAIN && edge) zero_unowned(vf, kb, g, wave_lo, k_len);
-          f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-          for (int ks = 0; ks < KEY_SLABS; ++ks) acc = mma_slab(vf[ks], pf[qt][ks], acc);
-          f32x4& A = As[qt][dt];
-          if (PLAIN || some[qt]) {
-            A.x = fold1(A.x, acc.x, ca[qt], cb[qt]);
-            A.y = fold1(A.y, acc.y, ca[qt], cb[qt]);
-            A.z = fold1(A.z, acc.z, ca[qt], cb[qt]);
-            A.w = fold1(A.w, acc.w, ca[qt], cb[qt]);
-          }
-        }
-      };
-#pragma unroll
-      for (int qt = 0; qt < QT; ++qt) {
-        if (!edge && all_some[qt]) pv(std::true_type{}, qt);
-        else pv(std::false_type{}, qt);
-      }
-    }
-    if ((t + 1) % SEG_TILES == 0 || t == tile_hi) {        // the segment is complete
-#pragma unroll
-      for (int qt = 0; qt < QT; ++qt) {
-        fold<NDT>(M[qt], L[qt], ACC[qt], Ms[qt], Ls[qt], As[qt]);
-        Ms[qt] = -INFINITY;
-        Ls[qt] = 0.f;
-#pragma unroll
-        for (int dt = 0; dt < NDT; ++dt) As[qt][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-      }
-    }
-  }
-#pragma unroll
-  for (int qt = 0; qt < QT; ++qt) {
-    if (row_ok[qt]) {
-      const float inv = L[qt] > 0.f ? 1.0f / L[qt] : 0.f;
-      elem_t* orow = a.out + ((int64_t)tok[qt] * a.nq + head) * a.d;
+      __builtin_amdgcn_s_setprio(0);
+      __builtin_amdgcn_sched_barrier(0);
+      // ---- the row's new maximum, its probabilities, its sums so far under the new maximum ----
+      const bool full = rows_wave >= 16 && kb + TILE_KEYS - 1 <= pos_wave &&
+                        kb >= (a.window > 0 ? max(0, pos_wave + 15 - a.window + 1) : 0);
+      frag_t pf[KEY_SLABS];
+      float ca;
+      const bool fresh = !(Ms > -INFINITY);
+      tile_probs(sc, kb, g, row_ok, lo, pos, a.scale_log2, full, Ms, Ls, ca, pf);
+      scale_state<NDT>(As, ca, fresh);
+      __builtin_amdgcn_sched_barrier(0);
+      // ---- P V onto the segment's sums, column block by column block ----
+      __builtin_amdgcn_s_setprio(1);
 #pragma unroll
       for (int dt = 0; dt < NDT; ++dt) {
-        const float o[4] = {ACC[qt][dt].x * inv, ACC[qt][dt].y * inv, ACC[qt][dt].z * inv, ACC[qt][dt].w * inv};
-        elem_t* p = orow + dt * 16 + 4 * g;
+        const int vrow = dt * 16 + r16;
+        const unsigned char* vr = vl + vrow * VRB;
+        const int sw = val_swz(vrow);
+        frag_t vf[KEY_SLABS];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) p[i] = from_f32<elem_t>(o[i]);
+        for (int ks = 0; ks < KEY_SLABS; ++ks) vf[ks] = *reinterpret_cast<const frag_t*>(vr + (((ks * 4 + g) ^ sw) << 4));
+#pragma unroll
+        for (int ks = 0; ks < KEY_SLABS; ++ks) As[dt] = mma_slab(vf[ks], pf[ks], As[dt]);
       }
+      __builtin_amdgcn_s_setprio(0);
+    }
+    if ((t + 1) % SEG_TILES == 0 || t == tile_hi) {        // the segment is complete
+      fold<NDT>(M, L, ACC, Ms, Ls, As);
+      Ms = -INFINITY;
+      Ls = 0.f;
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt) As[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+  }
+  if (row_ok) {
+    const float inv = L > 0.f ? 1.0f / L : 0.f;
+    elem_t* orow = a.out + ((int64_t)tok * a.nq + head) * a.d;
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) {
+      const float o[4] = {ACC[dt].x * inv, ACC[dt].y * inv, ACC[dt].z * inv, ACC[dt].w * inv};
+      elem_t* op = orow + dt * 16 + 4 * g;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) op[i] = from_f32<elem_t>(o[i]);
     }
   }
 }
 
-// Decoded tokens: an item is one token; the 16 rows of a wave are up to 16 q
-// heads of one kv head.  Workgroup = one segment, wave = one tile of it.
+// Decoded tokens: an item is one token; the 16 rows of a wave are up to 16 q heads of one kv head.  A wave takes
+// a segment, tile after tile, and asks for a tile's fragments when it needs them: for head and element sizes whose
+// fragments of two tiles do not fit a wave's registers.  The waves of a workgroup are neighbouring segments.
+#define PLAIN_WAVES 4
 template <int DPAD, bool V_LATE>
-__global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
+__global__ __launch_bounds__(64 * PLAIN_WAVES) void attn_decode_plain_kernel(AttnArgs a) {
   constexpr int NDT = DPAD / 16, NQS = DPAD / VK_SLAB;
-  extern __shared__ __attribute__((aligned(16))) float smem[];
-  float (*s_acc)[16][DPAD] = reinterpret_cast<float (*)[16][DPAD]>(smem);
-  float (*s_ml)[16][2] = reinterpret_cast<float (*)[16][2]>(smem + SEG_TILES * 16 * DPAD);
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int G = a.nq / a.nkv, HT = (G + 15) >> 4;
   const int kvh = blockIdx.y / HT, ht = blockIdx.y - kvh * HT;
-  const int seg = blockIdx.z;
+  const int seg = blockIdx.z * PLAIN_WAVES + wave;
   const int seq = a.items[2 * blockIdx.x], q_off = a.items[2 * blockIdx.x + 1];
   const int q_begin = a.cu_q[seq], q_len = a.cu_q[seq + 1] - q_begin;
   const int k_len = a.k_len[seq];
   const int tok = q_begin + q_off;
   const int pos = k_len - q_len + q_off;
   const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
-  const int tile_lo = lo / TILE_KEYS, tile_hi = pos / TILE_KEYS;
-  if (seg < tile_lo / SEG_TILES || seg > tile_hi / SEG_TILES) return;   // whole workgroup
+  const int t0 = max(lo / TILE_KEYS, seg * SEG_TILES), t1 = min(pos / TILE_KEYS, seg * SEG_TILES + SEG_TILES - 1);
+  if (t0 > t1) return;   // whole wave; no barrier follows
 
   RowCtx c;
   init_ctx(c, a, seq, kvh, k_len);
   c.r16 = lane & 15;
   c.g = lane >> 4;
-  const int nvalid = min(16, G - ht * 16);
-  c.row_ok = c.r16 < nvalid;
+  c.row_ok = c.r16 < min(16, G - ht * 16);
   c.pos = pos;
   c.lo = lo;
   c.wave_lo = lo;
   const int head = kvh * G + ht * 16 + c.r16;
-  const int t = seg * SEG_TILES + wave;
-  float m_t = -INFINITY, l_t = 0.f;
-  if (t >= tile_lo && t <= tile_hi) {
-    frag_t qf[NQS];
-    load_q<NQS>(a, tok, head, c.row_ok, c.g, qf);
-    f32x4 acc[NDT];
-    tile_partial<NDT, NQS, V_LATE>(c, qf, t * TILE_KEYS, m_t, l_t, acc);
-#pragma unroll
-    for (int dt = 0; dt < NDT; ++dt)
-      if (dt * 16 < a.d) *reinterpret_cast<f32x4*>(&s_acc[wave][c.r16][dt * 16 + 4 * c.g]) = acc[dt];
-  }
-  if (c.g == 0) {
-    s_ml[wave][c.r16][0] = m_t;
-    s_ml[wave][c.r16][1] = l_t;
-  }
-  __syncthreads();
-  // Fold the segment's tiles: thread (row, column group) owns DPAD/16 columns.
-  const int row = threadIdx.x >> 4, cg = threadIdx.x & 15;
-  if (row >= nvalid) return;
+  frag_t qf[NQS];
+  load_q<NQS>(a, tok, head, c.row_ok, c.g, qf);
   float M = -INFINITY, L = 0.f;
-  float ACC[NDT];
+  f32x4 ACC[NDT];
 #pragma unroll
-  for (int i = 0; i < NDT; ++i) ACC[i] = 0.f;
-#pragma unroll
-  for (int w = 0; w < SEG_TILES; ++w) {
-    const float m = s_ml[w][row][0], l = s_ml[w][row][1];
-    if (m > -INFINITY) {
-      float Mn, ca, cb;
-      fold_scales(M, m, Mn, ca, cb);
-#pragma unroll
-      for (int i = 0; i < NDT; ++i) ACC[i] = fold1(ACC[i], s_acc[w][row][cg * NDT + i], ca, cb);
-      L = fold1(L, l, ca, cb);
-      M = Mn;
-    }
-  }
-  const int64_t prow = ((int64_t)blockIdx.x * a.nq + (kvh * G + ht * 16 + row)) * a.nseg + seg;
-  if (cg == 0) {
+  for (int dt = 0; dt < NDT; ++dt) ACC[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int t = t0; t <= t1; ++t) tile_step<NDT, NQS, V_LATE>(c, qf, t * TILE_KEYS, M, L, ACC);
+  if (!c.row_ok) return;
+  const int64_t prow = ((int64_t)blockIdx.x * a.nq + head) * a.nseg + seg;
+  if (c.g == 0) {
     a.part_ml[2 * prow] = M;
     a.part_ml[2 * prow + 1] = L;
   }
   if (M > -INFINITY) {
 #pragma unroll
-    for (int i = 0; i < NDT; ++i)
-      if (cg * NDT + i < a.d) a.part_acc[prow * a.d + cg * NDT + i] = ACC[i];
+    for (int dt = 0; dt < NDT; ++dt)
+      if (dt * 16 < a.d) *reinterpret_cast<f32x4*>(&a.part_acc[prow * a.d + dt * 16 + 4 * c.g]) = ACC[dt];
   }
 }
 
-// Decoded tokens with many keys: a wave takes a whole segment, tile after tile, and folds in
+// Decoded tokens with many keys: a wave takes a whole segment, tile after tile, its state in
 // registers.  The keys of the next tile are asked for as soon as this tile's scores have left
 // their registers, the next values once this tile's product is done, so that a wave has half a
 // tile or more in flight all the time and the tables and the q rows are read once per segment.
@@ -758,33 +731,12 @@ __global__ __launch_bounds__(64 * SEG_WAVES, 2) void attn_decode_seg_kernel(Attn
     // Every row of a decoded token's wave stands at the same position: the masks are needed in the
     // tiles that hold the window's edge or the token itself only.
     const bool full = kb >= lo && kb + TILE_KEYS - 1 <= pos;
-    float m_t, l_t;
     frag_t pf[KEY_SLABS];
-    tile_softmax(sc, kb, c.g, c.row_ok, lo, pos, c.scale_log2, full, m_t, l_t, pf);
-    // The tile's product and its fold, head column by head column, so that the tile's own sums
-    // never stand in registers all at once (fold() does the same arithmetic on whole tiles).
-    const bool seen = m_t > -INFINITY;
-    float Mn, ca, cb;
-    fold_scales(M, m_t, Mn, ca, cb);
-    if (kb + TILE_KEYS > c.k_len || kb < c.wave_lo) {
-#pragma unroll
-      for (int dt = 0; dt < NDT; ++dt)
-        if (EXACT || dt * 16 < c.d) zero_unowned(vf[dt], kb, c.g, c.wave_lo, c.k_len);
-    }
-#pragma unroll
-    for (int dt = 0; dt < NDT; ++dt) {
-      if (EXACT || dt * 16 < c.d) {
-        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int ks = 0; ks < KEY_SLABS; ++ks) acc = mma_slab(vf[dt][ks], pf[ks], acc);
-        ACC[dt].x = seen ? fold1(ACC[dt].x, acc.x, ca, cb) : ACC[dt].x;
-        ACC[dt].y = seen ? fold1(ACC[dt].y, acc.y, ca, cb) : ACC[dt].y;
-        ACC[dt].z = seen ? fold1(ACC[dt].z, acc.z, ca, cb) : ACC[dt].z;
-        ACC[dt].w = seen ? fold1(ACC[dt].w, acc.w, ca, cb) : ACC[dt].w;
-      }
-    }
-    L = seen ? fold1(L, l_t, ca, cb) : L;
-    M = seen ? Mn : M;
+    float ca;
+    const bool fresh = !(M > -INFINITY);
+    tile_probs(sc, kb, c.g, c.row_ok, lo, pos, c.scale_log2, full, M, L, ca, pf);
+    scale_state<NDT>(ACC, ca, fresh);
+    tile_pv<NDT, EXACT>(c, kb, vf, pf, ACC);
     __builtin_amdgcn_sched_barrier(0);
     if (more) load_values<NDT, EXACT>(c, kb + TILE_KEYS, vf);
     __builtin_amdgcn_sched_barrier(0);
@@ -808,11 +760,10 @@ __global__ __launch_bounds__(64 * SEG_WAVES, 2) void attn_decode_seg_kernel(Attn
 
 // The same with two waves a segment, for steps with so few (token, kv head, segment) triples that a wave each
 // leaves most of the chip idle and every wave waits for its four tiles one after the other: the first wave
-// takes the first half of the segment's tiles, the second wave the rest.  The second wave starts from an empty
-// state, which its first tile fills with that tile's own sums exactly (a fold onto nothing scales by 0 and 1);
-// when the first wave has left its state in LDS, the second folds its own onto it (the fold of that tile onto
-// the tiles before it, as the one wave computes it) and goes on with its other tile: the same bits, and the
-// loads of both halves in flight together.
+// takes the first half of the segment's tiles, the second wave the rest.  The second wave asks for its first
+// tile's keys and values at once and computes that tile's scores, which need no state; when the first wave has
+// left the segment's state in LDS, the second takes it and goes on from there as the one wave would: the same
+// bits, and the loads of both halves in flight together.
 template <int DPAD, bool EXACT>
 __global__ __launch_bounds__(128, 2) void attn_decode_pair_kernel(AttnArgs a) {
   constexpr int NDT = DPAD / 16, NQS = DPAD / VK_SLAB;
@@ -855,67 +806,45 @@ __global__ __launch_bounds__(128, 2) void attn_decode_pair_kernel(AttnArgs a) {
   f32x4 ACC[NDT];
 #pragma unroll
   for (int dt = 0; dt < NDT; ++dt) ACC[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  auto tile = [&](int t, bool more) {
-    const int kb = t * TILE_KEYS;
-    float sc[S_PER_LANE];
+  float sc[S_PER_LANE];
+  // A tile's scores, and its successor's keys asked for.
+  auto front = [&](int t, bool more) {
     tile_scores<NQS, EXACT>(c, kf, qf, sc);
     __builtin_amdgcn_sched_barrier(0);
-    if (more) load_keys<NQS, EXACT>(c, kb + TILE_KEYS, kf);
+    if (more) load_keys<NQS, EXACT>(c, (t + 1) * TILE_KEYS, kf);
     __builtin_amdgcn_sched_barrier(0);
+  };
+  // The tile onto the state, and its successor's values asked for.
+  auto back = [&](int t, bool more) {
+    const int kb = t * TILE_KEYS;
     const bool full = kb >= lo && kb + TILE_KEYS - 1 <= pos;
-    float m_t, l_t;
     frag_t pf[KEY_SLABS];
-    tile_softmax(sc, kb, c.g, c.row_ok, lo, pos, c.scale_log2, full, m_t, l_t, pf);
-    const bool seen = m_t > -INFINITY;
-    float Mn, ca, cb;
-    fold_scales(M, m_t, Mn, ca, cb);
-    if (kb + TILE_KEYS > c.k_len || kb < c.wave_lo) {
-#pragma unroll
-      for (int dt = 0; dt < NDT; ++dt)
-        if (EXACT || dt * 16 < c.d) zero_unowned(vf[dt], kb, c.g, c.wave_lo, c.k_len);
-    }
-#pragma unroll
-    for (int dt = 0; dt < NDT; ++dt) {
-      if (EXACT || dt * 16 < c.d) {
-        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int ks = 0; ks < KEY_SLABS; ++ks) acc = mma_slab(vf[dt][ks], pf[ks], acc);
-        ACC[dt].x = seen ? fold1(ACC[dt].x, acc.x, ca, cb) : ACC[dt].x;
-        ACC[dt].y = seen ? fold1(ACC[dt].y, acc.y, ca, cb) : ACC[dt].y;
-        ACC[dt].z = seen ? fold1(ACC[dt].z, acc.z, ca, cb) : ACC[dt].z;
-        ACC[dt].w = seen ? fold1(ACC[dt].w, acc.w, ca, cb) : ACC[dt].w;
-      }
-    }
-    L = seen ? fold1(L, l_t, ca, cb) : L;
-    M = seen ? Mn : M;
+    float ca;
+    const bool fresh = !(M > -INFINITY);
+    tile_probs(sc, kb, c.g, c.row_ok, lo, pos, c.scale_log2, full, M, L, ca, pf);
+    scale_state<NDT>(ACC, ca, fresh);
+    tile_pv<NDT, EXACT>(c, kb, vf, pf, ACC);
     __builtin_amdgcn_sched_barrier(0);
     if (more) load_values<NDT, EXACT>(c, kb + TILE_KEYS, vf);
     __builtin_amdgcn_sched_barrier(0);
   };
-  // At most two tiles a wave.  The second wave's first tile starts from nothing: its state is then that tile's
-  // own sums; it waits for the first wave's state and folds its own onto it.
-  tile(t0, t0 < t1);
+  // At most two tiles a wave.
+  front(t0, t0 < t1);
   if (wave == 1) {
-    __syncthreads();
-    const float Ma = hand_ml[0][lane], La = hand_ml[1][lane];
-    const bool seen = M > -INFINITY;
-    float Mn, ca, cb;
-    fold_scales(Ma, M, Mn, ca, cb);
-#pragma unroll
-    for (int dt = 0; dt < NDT; ++dt) {
-      const f32x4 A = hand_acc[dt][lane];
-      ACC[dt].x = seen ? fold1(A.x, ACC[dt].x, ca, cb) : A.x;
-      ACC[dt].y = seen ? fold1(A.y, ACC[dt].y, ca, cb) : A.y;
-      ACC[dt].z = seen ? fold1(A.z, ACC[dt].z, ca, cb) : A.z;
-      ACC[dt].w = seen ? fold1(A.w, ACC[dt].w, ca, cb) : A.w;
-    }
-    L = seen ? fold1(La, L, ca, cb) : La;
-    M = seen ? Mn : Ma;
-  }
-  if (t0 < t1) tile(t1, false);
-  if (wave == 0 && paired) {
-    // The first half's state, for the second wave (every lane its own part: the same lanes hold the same rows
+    // The segment's state as the first wave left it (every lane its own part: the same lanes hold the same rows
     // and columns in both waves).
+    __syncthreads();
+    M = hand_ml[0][lane];
+    L = hand_ml[1][lane];
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) ACC[dt] = hand_acc[dt][lane];
+  }
+  back(t0, t0 < t1);
+  if (t0 < t1) {
+    front(t1, false);
+    back(t1, false);
+  }
+  if (wave == 0 && paired) {
     hand_ml[0][lane] = M;
     hand_ml[1][lane] = L;
 #pragma unroll
@@ -934,98 +863,6 @@ __global__ __launch_bounds__(128, 2) void attn_decode_pair_kernel(AttnArgs a) {
     for (int dt = 0; dt < NDT; ++dt)
       if (EXACT || dt * 16 < a.d) *reinterpret_cast<f32x4*>(&a.part_acc[prow * a.d + dt * 16 + 4 * c.g]) = ACC[dt];
   }
-}
-
-// Decoded tokens, all keys of a token in one workgroup: for batches that fill the chip without a
-// split over segments, and contexts whose tile results fit LDS.  Eight waves take the tiles in turn
-// (wave w: tiles first + w, first + w + 8, ...), every tile's (m, l, acc) goes to LDS, and after one
-// barrier the threads fold them exactly as attn_decode and attn_combine do together: tiles into
-// their segment in order, segments into the total in order.  No scratch buffer, no second launch.
-#define WHOLE_WAVES 8
-template <int DPAD>
-__global__ __launch_bounds__(64 * WHOLE_WAVES) void attn_decode_whole_kernel(AttnArgs a, int tiles_cap) {
-  constexpr int NDT = DPAD / 16, NQS = DPAD / VK_SLAB;
-  extern __shared__ __attribute__((aligned(16))) float smem[];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int G = a.nq / a.nkv, HT = (G + 15) >> 4;
-  const int kvh = blockIdx.y / HT, ht = blockIdx.y - kvh * HT;
-  const int nvalid = min(16, G - ht * 16);
-  float* s_acc = smem;                                         // [tiles_cap][nvalid][DPAD]
-  float* s_ml = smem + (size_t)tiles_cap * nvalid * DPAD;      // [tiles_cap][nvalid][2]
-  const int seq = a.items[2 * blockIdx.x], q_off = a.items[2 * blockIdx.x + 1];
-  const int q_begin = a.cu_q[seq], q_len = a.cu_q[seq + 1] - q_begin;
-  const int k_len = a.k_len[seq];
-  const int tok = q_begin + q_off;
-  const int pos = k_len - q_len + q_off;
-  const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
-  const int tile_lo = lo / TILE_KEYS, tile_hi = pos / TILE_KEYS;   // tile_hi - tile_lo < tiles_cap (host)
-
-  RowCtx c;
-  init_ctx(c, a, seq, kvh, k_len);
-  c.r16 = lane & 15;
-  c.g = lane >> 4;
-  c.row_ok = c.r16 < nvalid;
-  c.pos = pos;
-  c.lo = lo;
-  c.wave_lo = lo;
-  const int head0 = kvh * G + ht * 16;
-  frag_t qf[NQS];
-  load_q<NQS>(a, tok, head0 + c.r16, c.row_ok, c.g, qf);
-  for (int t = tile_lo + wave; t <= tile_hi; t += WHOLE_WAVES) {
-    float m_t, l_t;
-    f32x4 acc[NDT];
-    tile_partial<NDT, NQS, false>(c, qf, t * TILE_KEYS, m_t, l_t, acc);
-    if (c.row_ok) {
-      float* dst = s_acc + ((size_t)(t - tile_lo) * nvalid + c.r16) * DPAD;
-#pragma unroll
-      for (int dt = 0; dt < NDT; ++dt)
-        if (dt * 16 < a.d) *reinterpret_cast<f32x4*>(dst + dt * 16 + 4 * c.g) = acc[dt];
-      if (c.g == 0) {
-        s_ml[((t - tile_lo) * nvalid + c.r16) * 2] = m_t;
-        s_ml[((t - tile_lo) * nvalid + c.r16) * 2 + 1] = l_t;
-      }
-    }
-  }
-  __syncthreads();
-  // Thread (row, column group) owns DPAD/16 columns of one row.
-  const int row = threadIdx.x >> 4, cg = threadIdx.x & 15;
-  if (row >= nvalid) return;
-  float M = -INFINITY, L = 0.f;
-  float ACC[NDT];
-#pragma unroll
-  for (int i = 0; i < NDT; ++i) ACC[i] = 0.f;
-  for (int seg = tile_lo / SEG_TILES; seg <= tile_hi / SEG_TILES; ++seg) {
-    float Ms = -INFINITY, Ls = 0.f;
-    float As[NDT];
-#pragma unroll
-    for (int i = 0; i < NDT; ++i) As[i] = 0.f;
-    const int t_end = min(tile_hi, seg * SEG_TILES + SEG_TILES - 1);
-    for (int t = max(tile_lo, seg * SEG_TILES); t <= t_end; ++t) {
-      const int e = (t - tile_lo) * nvalid + row;
-      const float m = s_ml[2 * e], l = s_ml[2 * e + 1];
-      if (m > -INFINITY) {
-        float Mn, ca, cb;
-        fold_scales(Ms, m, Mn, ca, cb);
-#pragma unroll
-        for (int i = 0; i < NDT; ++i) As[i] = fold1(As[i], s_acc[(size_t)e * DPAD + cg * NDT + i], ca, cb);
-        Ls = fold1(Ls, l, ca, cb);
-        Ms = Mn;
-      }
-    }
-    if (Ms > -INFINITY) {
-      float Mn, ca, cb;
-      fold_scales(M, Ms, Mn, ca, cb);
-#pragma unroll
-      for (int i = 0; i < NDT; ++i) ACC[i] = fold1(ACC[i], As[i], ca, cb);
-      L = fold1(L, Ls, ca, cb);
-      M = Mn;
-    }
-  }
-  const float inv = L > 0.f ? 1.0f / L : 0.f;
-  elem_t* orow = a.out + ((int64_t)tok * a.nq + head0 + row) * a.d;
-#pragma unroll
-  for (int i = 0; i < NDT; ++i)
-    if (cg * NDT + i < a.d) orow[cg * NDT + i] = from_f32<elem_t>(ACC[i] * inv);
 }
 
 // Folds the segment results of one (token, head) in ascending segment order.
@@ -1148,24 +985,24 @@ int vk_paged_attention(elem_t* out, const elem_t* q, const elem_t* kc, const ele
   if (mode == 0 && vk_attn_prefill_shares_tiles(d, P)) {
     VK_REQUIRE((int64_t)n_items * (ITEM_ROWS / 16) * nq < (1ll << 31), "attention: too many prompt items");
     const size_t smem = (size_t)4 * TILE_KEYS * d * sizeof(elem_t);
-#define PREFILL_LDS(DP, QT, NW)                                                                      \
+#define PREFILL_LDS(DP, NW)                                                                          \
   do {                                                                                               \
     static bool raised = false;                                                                      \
     if (!raised) {                                                                                   \
-      (void)hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<DP, QT, NW>,                    \
+      (void)hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<DP, NW>,                        \
                                 hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);             \
       raised = true;                                                                                 \
     }                                                                                                \
-    attn_prefill_lds_kernel<DP, QT, NW><<<n_items * (ITEM_ROWS / (16 * QT * NW)) * nq, 64 * NW, smem, st>>>(a, n_items); \
+    attn_prefill_lds_kernel<DP, NW><<<n_items * (ITEM_ROWS / (16 * NW)) * nq, 64 * NW, smem, st>>>(a, n_items); \
   } while (0)
     // Eight waves of one row tile each measured best on long contexts (MI355X, head size 128); four
-    // waves are a few per cent better on short ones.  Two row tiles per wave (QT = 2) would halve the
-    // LDS traffic but need more than the 256 registers that two waves per SIMD leave: with spills or
+    // waves are a few per cent better on short ones.  Two row tiles per wave would halve the LDS
+    // traffic but need more than the 256 registers that two waves per SIMD leave: with spills or
     // with one wave per SIMD they measured 40 % slower.
     const int v = vk_prefill_variant;
-    if (d == 64) { if (v == 14) PREFILL_LDS(64, 1, 4); else PREFILL_LDS(64, 1, 8); }
-    else if (d == 128) { if (v == 14) PREFILL_LDS(128, 1, 4); else PREFILL_LDS(128, 1, 8); }
-    else { if (v == 14) PREFILL_LDS(256, 1, 4); else PREFILL_LDS(256, 1, 8); }
+    if (d == 64) { if (v == 14) PREFILL_LDS(64, 4); else PREFILL_LDS(64, 8); }
+    else if (d == 128) { if (v == 14) PREFILL_LDS(128, 4); else PREFILL_LDS(128, 8); }
+    else { if (v == 14) PREFILL_LDS(256, 4); else PREFILL_LDS(256, 8); }
 #undef PREFILL_LDS
     return vk_check_launch("attention (prompt rows, shared tiles)");
   }
@@ -1180,47 +1017,14 @@ int vk_paged_attention(elem_t* out, const elem_t* q, const elem_t* kc, const ele
     return vk_check_launch("attention (prompt rows)");
   }
   VK_REQUIRE(nseg > 0 && nseg <= 65535 && scratch != nullptr, "attention: decode needs nseg in 1..65535 and scratch");
-  // A wave per segment where a wave's registers hold two tiles' fragments (a tile's keys, or its
-  // values, are 32 * head size * element size bytes of them): see below.  The other two kernels
-  // are for the larger head and element sizes.
+  // A wave per segment with the next tile's fragments in flight where a wave's registers hold two tiles'
+  // fragments (a tile's keys, or its values, are 32 * head size * element size bytes of them); the kernel that
+  // asks for a tile's fragments when it needs them is for the larger head and element sizes.
   const bool seg_fits = sizeof(elem_t) * vk_dpad(d) <= 256;
-  {
-    // One workgroup per (token, kv head) when there are enough of them to fill the chip's memory pipes
-    // and the tiles' results fit LDS; else the keys are split over workgroups by segment (below).
-    // Measured on MI355X at 2,060 keys and head size 128: 64 tokens 110 against 117 us, 16 tokens 45
-    // against 35 us (a wave walks its tiles one after the other, so few workgroups are latency-bound).
-    const int HT = (G + 15) / 16, rows = G < 16 ? G : 16;
-    const int tiles_cap = nseg * SEG_TILES;
-    const size_t smem = (size_t)tiles_cap * rows * (vk_dpad(d) + 2) * sizeof(float);
-    const int64_t wgs = (int64_t)n_items * nkv * HT;
-    const bool whole = vk_decode_variant == 1 || (vk_decode_variant == 0 && !seg_fits && wgs >= 448 && smem <= 96 * 1024);
-    if (whole && smem <= 150 * 1024) {
-      const dim3 grid(n_items, nkv * HT);
-      VK_REQUIRE(grid.y <= 65535, "attention: too many heads");
-#define DECODE_WHOLE(DP)                                                                             \
-  do {                                                                                               \
-    static bool raised = false;                                                                      \
-    if (!raised) {                                                                                   \
-      (void)hipFuncSetAttribute((const void*)attn_decode_whole_kernel<DP>,                           \
-                                hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);             \
-      raised = true;                                                                                 \
-    }                                                                                                \
-    attn_decode_whole_kernel<DP><<<grid, 64 * WHOLE_WAVES, smem, st>>>(a, tiles_cap);                \
-  } while (0)
-      if (d <= 64) DECODE_WHOLE(64);
-      else if (d <= 128) DECODE_WHOLE(128);
-      else DECODE_WHOLE(256);
-#undef DECODE_WHOLE
-      return vk_check_launch("attention (decoded rows, whole)");
-    }
-  }
   a.part_ml = scratch;
   a.part_acc = scratch + (((int64_t)n_items * nq * nseg * 2 + 3) & ~(int64_t)3);
   const dim3 grid(n_items, nkv * ((G + 15) / 16), nseg);
   VK_REQUIRE(grid.y <= 65535 && nq <= 65535, "attention: too many heads");
-  // Measured on MI355X, bfloat16, head size 128: from one token of 300 keys (15.5 against 17.2 us)
-  // over 8 tokens of 2,060 keys (19 against 25 us) to 64 tokens of 8,231 keys (446 against 506 us)
-  // the wave per segment is never slower than the kernel below, nor than the one above.
   static_assert(SEG_TILES == 4, "the pair kernel gives a wave two tiles at most");
   // Two waves a segment while there are no more segments in work than one and a quarter per compute unit
   // (measured on MI355X, head size 128, 8 kv heads, with the fold of the segments; a wave against two waves a
@@ -1260,22 +1064,19 @@ int vk_paged_attention(elem_t* out, const elem_t* q, const elem_t* kc, const ele
     attn_combine_kernel<<<dim3(n_items, nq), 64, 0, st>>>(a);
     return vk_check_launch("attention (combine)");
   }
-#define DECODE(DP, LATE)                                                                             \
-  do {                                                                                               \
-    const size_t smem = (size_t)SEG_TILES * 16 * (DP + 2) * sizeof(float);                           \
-    if (smem > 48 * 1024)                                                                            \
-      (void)hipFuncSetAttribute((const void*)attn_decode_kernel<DP, LATE>,                           \
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);              \
-    attn_decode_kernel<DP, LATE><<<grid, 256, smem, st>>>(a);                                        \
-  } while (0)
-  // With few workgroups a wave asks for keys and values together; with many, the values wait until
-  // the keys' registers are free, so that more waves fit a SIMD (measured on MI355X: the two cross
-  // between 8 and 64 tokens of 2,000 keys).
+  // With few waves a wave asks for keys and values together; with many, the values wait until the keys'
+  // registers are free, so that more waves fit a SIMD.
+  const dim3 pgrid(grid.x, grid.y, (nseg + PLAIN_WAVES - 1) / PLAIN_WAVES);
   const bool late = (int64_t)grid.x * grid.y * grid.z > 1024;
-  if (d <= 64) { if (late) DECODE(64, true); else DECODE(64, false); }
-  else if (d <= 128) { if (late) DECODE(128, true); else DECODE(128, false); }
-  else { if (late) DECODE(256, true); else DECODE(256, false); }
-#undef DECODE
+#define DECODE_PLAIN(DP)                                                                    \
+  do {                                                                                      \
+    if (late) attn_decode_plain_kernel<DP, true><<<pgrid, 64 * PLAIN_WAVES, 0, st>>>(a);    \
+    else attn_decode_plain_kernel<DP, false><<<pgrid, 64 * PLAIN_WAVES, 0, st>>>(a);        \
+  } while (0)
+  if (d <= 64) DECODE_PLAIN(64);
+  else if (d <= 128) DECODE_PLAIN(128);
+  else DECODE_PLAIN(256);
+#undef DECODE_PLAIN
   if (vk_check_launch("attention (decoded rows)")) return 1;
   attn_combine_kernel<<<dim3(n_items, nq), 64, 0, st>>>(a);
   return vk_check_launch("attention (combine)");

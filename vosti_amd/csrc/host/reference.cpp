@@ -5,8 +5,10 @@
 //   * projections: K in chunks of 512 from 0; within a chunk the products are added to a sum that starts
 //     at zero, slab (64 bytes of a row) after slab, and inside a slab in the order in which mma_slab
 //     feeds the matrix unit; the chunk sums are added to a zero total in chunk order (gemm.hip);
-//   * attention: keys in tiles of 64 at absolute positions, each tile reduced on its own, tiles folded
-//     into segments of four, segments into the total, all in ascending order (attention.hip).
+//   * attention: keys in tiles of 64 at absolute positions; a segment of four tiles takes its tiles in, ascending,
+//     onto a running state (a reference maximum that moves when the tile's exceeds it by more than 2^8, the sums
+//     so far scaled when it moves, the tile's products added); the segments are folded into the total in ascending
+//     order (attention.hip).
 // Storage is float everywhere; `bf16` != 0 rounds every value that the kernels store in the element
 // type to bfloat16 (round to nearest even), which is where the reference engine rounds too
 // (every formula cites its source in the kernel's own file).
@@ -44,13 +46,13 @@ constexpr int SEG_TILES = 4;
 // 2^x as the fold and the probabilities use it.
 inline float exp2_ref(float x) { return std::exp2(x); }
 
-struct Partial {                 // (m, l, acc[d]) of a tile, a segment or a row
+struct Partial {                 // (m, l, acc[d]) of a segment or a row
   float m = -INFINITY, l = 0.f;
   std::vector<float> acc;
   explicit Partial(int d) : acc(d, 0.f) {}
 };
 
-// state <- fold of a non-empty partial: M' = max(M, m); X' = fma(x, 2^(m - M'), X * 2^(M - M')).
+// state <- fold of a non-empty segment: M' = max(M, m); X' = fma(x, 2^(m - M'), X * 2^(M - M')).
 void fold(Partial& S, const Partial& p) {
   if (!(p.m > -INFINITY)) return;
   const float Mn = std::fmax(S.m, p.m);
@@ -189,7 +191,7 @@ void vh_ref_qkv_post(float* q_out, float* kc, float* vc, const float* qkv, const
 
 // Causal grouped-query attention over the paged cache for every row of every sequence.  Row r of a
 // sequence with q_len rows and k_len keys stands at position k_len - q_len + r and sees the keys
-// max(0, p - window + 1) .. p (all from 0 without a window).  Tile, segment and total as in attention.hip.
+// max(0, p - window + 1) .. p (all from 0 without a window).  Tiles, segments and total as in attention.hip.
 void vh_ref_paged_attention(float* out, const float* q, const float* kc, const float* vc, const int32_t* block_table,
                             int bt_stride, const int32_t* cu_q, const int32_t* k_len, int S, int nq, int nkv, int d,
                             int P, int window, float scale, int bf16) {
@@ -212,7 +214,6 @@ void vh_ref_paged_attention(float* out, const float* q, const float* kc, const f
             for (int t = seg * SEG_TILES; t < seg * SEG_TILES + SEG_TILES; ++t) {
               const int kb = t * TILE_KEYS;
               if (kb > pos || kb + TILE_KEYS <= lo) continue;
-              Partial tp(d);
               float mx = -INFINITY;
               for (int j = 0; j < TILE_KEYS; ++j) {
                 const int key = kb + j;
@@ -230,26 +231,30 @@ void vh_ref_paged_attention(float* out, const float* q, const float* kc, const f
                 sc[j] = acc;
                 mx = std::fmax(mx, acc);
               }
-              if (!(mx > -INFINITY)) continue;
-              tp.m = mx * c;
+              if (!(mx > -INFINITY)) continue;         // the row sees no key of the tile: its state stands
+              // The tile onto the segment's state: the new maximum, the sums so far under it, the tile's own added.
+              // The reference point moves only when the state is empty or the maximum grows by more than 2^8.
+              const float mt = mx * c;
+              const float Mn = (!(sp.m > -INFINITY) || mt > sp.m + 8.0f) ? mt : sp.m;
+              const float ca = exp2_ref(sp.m - Mn);      // 1 where the maximum stands, 0 while the state is empty
               float l = 0.f;
               for (int j = 0; j < TILE_KEYS; ++j) {
                 const int key = kb + j;
-                pr[j] = (key < lo || key > pos) ? 0.f : exp2_ref(std::fma(sc[j], c, -tp.m));
+                pr[j] = (key < lo || key > pos) ? 0.f : exp2_ref(std::fma(sc[j], c, -Mn));
                 l = l + pr[j];
               }
-              tp.l = l;
+              sp.l = std::fma(sp.l, ca, l);
+              sp.m = Mn;
               for (int i = 0; i < d; ++i) {
-                float a = 0.f;
+                float a = sp.acc[i] * ca;
                 for (int j = 0; j < TILE_KEYS; ++j) {
                   const int key = kb + j;
                   if (key < lo || key > pos) continue;
                   const float v = vc[(((int64_t)bt[key / P] * nkv + kvh) * d + i) * P + key % P];
                   a = a + v * store(pr[j], bf16);
                 }
-                tp.acc[i] = a;
+                sp.acc[i] = a;
               }
-              fold(sp, tp);
             }
             fold(total, sp);
           }
