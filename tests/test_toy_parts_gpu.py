@@ -35,6 +35,7 @@ def define_toy():
     @register_part("mixer", "toy_decay")
     class ToyDecay(Mixer):
         """state_t = sigmoid(a) * state_{t-1} + x_t, per request; y_t = state_t W^T."""
+        replayable = False           # forward walks the step's host numbers: a recording would repeat one step's slots
 
         def __init__(self, kernels, hidden_size):
             super().__init__(kernels)
@@ -314,8 +315,10 @@ def test_toy_generation_through_the_engine(toy_dir):
     from vosti_amd.sampling import SamplingParams
     prompts = toy_prompts()[:3]
     plain_model = PlainToy(toy_dir)
-    outs = Engine(toy_dir, dtype="float32", num_pages=40, page_size=8, max_num_seqs=3, max_num_batched_tokens=32).generate(
-        prompts, SamplingParams(max_tokens=10))
+    # Asked to record its decode steps, the engine does not: one of the toy's parts says that it cannot be replayed.
+    engine = Engine(toy_dir, dtype="float32", num_pages=40, page_size=8, max_num_seqs=3, max_num_batched_tokens=32, graphs=True)
+    outs = engine.generate(prompts, SamplingParams(max_tokens=10))
+    assert engine.runner.graph_stats["captured"] == 0 and engine.runner.graph_stats["replayed"] == 0
     for p, o in zip(prompts, outs):
         ids = list(p)
         for tok in o:

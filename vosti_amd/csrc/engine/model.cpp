@@ -293,6 +293,12 @@ void DecoderModel::random_weights(uint64_t seed) {
   loaded_ = true;
 }
 
+bool DecoderModel::replayable() {
+  for (Part* p : parts())
+    if (!p->replayable()) return false;
+  return true;
+}
+
 std::vector<CacheNeed> DecoderModel::cache_needs() {
   std::vector<CacheNeed> out;
   for (const ScheduleEntry& e : spec_.schedule) out.push_back(e.cache_from >= 0 ? CacheNeed{} : layers_[e.layer]->mixer().cache_need());

@@ -40,6 +40,7 @@ class DecoderModel {
   // Random weights from a seed, drawn on the GPU: every element is a function of (seed, tensor name, element
   // index), the values the Python package's random-weights mode stores for the same seed in the compute type.
   void random_weights(uint64_t seed);
+  bool replayable();                                        // every part's launches depend on arrays on the GPU alone
   std::vector<CacheNeed> cache_needs();                     // one per schedule entry (None if it reads another's)
   // ids int32 [T]; caches: one per schedule entry; want_rows int32 [R] -> logits [R, vocab].
   Tensor forward(const Tensor& ids, StepContext& ctx, std::vector<CacheEntry>& caches, const Tensor& want_rows);

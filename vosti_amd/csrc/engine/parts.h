@@ -84,6 +84,9 @@ class Part {
   virtual const char* step_inputs_key() const { return nullptr; }
   virtual void step_inputs(HostStep& step, std::vector<std::pair<std::string, HostArray>>& out) { (void)step; (void)out; }
   virtual int64_t workspace_floats(HostStep& step) { (void)step; return 0; }
+  // false: the part's launches depend on the step's host numbers (HostStep) and not only on the arrays on the
+  // GPU, so a recorded step would repeat one step's numbers; a model with such a part is never recorded.
+  virtual bool replayable() const { return true; }
 
  protected:
   Kernels& kernels;

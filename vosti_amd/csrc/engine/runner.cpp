@@ -82,7 +82,7 @@ struct ModelRunner::Captured {
 };
 
 ModelRunner::ModelRunner(DecoderModel& model, CachePool& pool, bool graphs, int max_graphs)
-    : model_(model), pool_(pool), k_(model.kernels()), graphs_(graphs), max_graphs_(std::max(1, max_graphs)) {
+    : model_(model), pool_(pool), k_(model.kernels()), graphs_(graphs && model.replayable()), max_graphs_(std::max(1, max_graphs)) {
   parts_ = model.parts();
   // What the parts want of every step: one provider per distinct kind of per-step arrays.
   std::set<std::string> keys;

@@ -80,7 +80,6 @@ class ModelRunner:
     def __init__(self, model, pool: CachePool, graphs: bool = False, max_graphs: int | None = None):
         self.model, self.pool, self.cache = model, pool, pool.manager
         self.kernels = model.kernels
-        self.graphs = graphs
         self.max_graphs = max(1, int(_max_graphs() if max_graphs is None else max_graphs))   # the least recently replayed goes first
         self._workspace: torch.Tensor | None = None
         self._seen: set[tuple] = set()
@@ -90,6 +89,7 @@ class ModelRunner:
         self.graph_stats = {"eager": 0, "captured": 0, "replayed": 0, "evicted": 0}
         # What the parts want of every step: one provider per distinct kind of per-step arrays.
         self._parts = list(model.parts())
+        self.graphs = graphs and all(part.replayable for part in self._parts)
         self._providers = {}
         for part in self._parts:
             if part.step_inputs_key is not None:

@@ -181,6 +181,10 @@ class Part:
         """float32 elements of ``ctx.workspace`` that this part's forward will ask for in this step."""
         return 0
 
+    # False: the part's launches depend on the step's host numbers (``ctx.host_*``) and not only on the arrays
+    # on the GPU, so a recorded step would repeat one step's numbers; a model with such a part is never recorded.
+    replayable = True
+
 
 class Norm(Part):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
