@@ -959,8 +959,9 @@ int vk_attn_prefill_shares_tiles(int d, int P) {
 // mode 1: each item is one token; the keys are split by segment over nseg workgroups (nseg must cover
 //   the longest sequence; scratch must hold vk_attn_scratch_floats(n_items, ...)) and folded by a
 //   second kernel; the kernel is chosen by shape.  modes 3, 4, 5, 7: the same through a named kernel
-//   (3: all keys of a token in one workgroup where LDS allows, 4: a wave per tile, 5: a wave per
-//   segment, 7: two waves per segment; tests and measurements; the same bits).
+//   (3 and 4: a wave per segment that asks for a tile's fragments when it needs them, the kernel for every
+//   shape; 5: a wave per segment with two tiles' fragments in registers; 7: two waves per segment; tests
+//   and measurements; the same bits).
 int vk_paged_attention(elem_t* out, const elem_t* q, const elem_t* kc, const elem_t* vc,
                        const int32_t* block_table, int bt_stride, const int32_t* cu_q, const int32_t* k_len,
                        const int32_t* items, int n_items, int mode, int nseg, float* scratch, int total_tokens,
