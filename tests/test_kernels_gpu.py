@@ -43,7 +43,8 @@ def test_gemm(dtype, M, N, K):
     got_t = k.gemm(a.cuda(), w.cuda(), kernel=2)
     torch.testing.assert_close(got_t.float().cpu(), ref.to(dtype).float(), **tol(dtype))
     if K % (64 if dtype == torch.bfloat16 else 32) == 0:
-        assert torch.equal(k.gemm(a.cuda(), w.cuda(), kernel=13), got_t), "64 weight rows per workgroup"
+        for code, rows in ((13, 64), (15, 96), (16, 160)):
+            assert torch.equal(k.gemm(a.cuda(), w.cuda(), kernel=code), got_t), f"{rows} weight rows per workgroup"
     if 64 < M <= 512 and K % 512 == 0:
         for code in (0, 8, 9, 10, 12):  # blocks of 64 (12: of 32) rows through the kernels that share activations through LDS
             assert torch.equal(k.gemm(a.cuda(), w.cuda(), kernel=code), got_t), code
@@ -68,6 +69,22 @@ def test_gemm(dtype, M, N, K):
     for r in {0, M // 2, M - 1}:
         one = k.gemm(a[r:r + 1].cuda(), w.cuda())
         assert torch.equal(one[0], got_t[r])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,N,K", [(2048, 5120, 512), (1024, 6144, 512), (4096, 5120, 576), (2000, 5000, 512), (1000, 6100, 640),
+                                   (2048, 10240, 256), (1536, 6144, 512)])
+def test_tile_width_chosen_by_rounds(dtype, M, N, K):
+    """Row and column counts at which the tile kernel is given 96 or 160 weight rows a workgroup instead of 128
+    (the last round of workgroups would otherwise run nearly empty), whole and with partial blocks in both
+    directions: the same bits as with 128, whichever width is named or chosen, and right."""
+    k = kern(dtype)
+    a, w = rand((M, K), dtype, 1), rand((N, K), dtype, 2, 0.1)
+    ref = (a.double() @ w.double().t()).float()
+    square = k.gemm(a.cuda(), w.cuda(), kernel=4)
+    torch.testing.assert_close(square.float().cpu(), ref.to(dtype).float(), **tol(dtype))
+    for code in (0, 2, 13, 15, 16):
+        assert torch.equal(k.gemm(a.cuda(), w.cuda(), kernel=code), square), code
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

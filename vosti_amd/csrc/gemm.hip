@@ -30,6 +30,8 @@
 //                       stages; a second accumulator set holds the total.  Optionally SwiGLU in the
 //                       epilogue.
 //   gemm_tiled          any M and K: the same tile through registers into LDS, predicated.
+#include <cmath>
+
 #include "common.h"
 #include "mma.h"
 #include "vec.h"
@@ -539,8 +541,10 @@ __device__ __forceinline__ unsigned lds_offset_of(const unsigned char* p) {
   return (unsigned)(unsigned long)((__attribute__((address_space(3))) const void*)p);
 }
 
-// FNW: 16-row weight fragments per wave, 4 (a workgroup takes 128 weight rows) or 2 (64: twice the
-// workgroups, for grids that would leave compute units with one workgroup or none).
+// FNW: 16-row weight fragments per wave, 2 to 5: a workgroup takes 32 FNW weight rows.  4 is the square tile; 2
+// gives twice the workgroups, for grids that would leave compute units with one workgroup or none; 3 and 5 are
+// for grids whose last round of workgroups would otherwise run nearly empty (pipe_fragments_by_rounds).  Six
+// would need more than the 256 registers of a wave.
 // One 4-byte load per lane whose value nobody reads: it brings the lane's 128-byte line into the second-level
 // cache ahead of the LDS-direct load that will want it.  `keep` is one register that every such load writes
 // (in order, so they may overlap) and that stays allocated to the end of the kernel.
@@ -557,7 +561,8 @@ template <int S, bool WHOLE, bool SWIGLU, int FNW = 4, int PFD = 0>
 __global__ __launch_bounds__(256, 2) void gemm_pipe_kernel(elem_t* __restrict__ out, const elem_t* __restrict__ act,
                                                         const elem_t* __restrict__ w, int M, int N, int K,
                                                         int64_t lda, int64_t ldo, int out_vec_ok, int band_w) {
-  static_assert(FNW == 4 || (FNW == 2 && !SWIGLU), "two or four weight fragments per wave");
+  static_assert(FNW >= 2 && FNW <= 5 && (FNW == 4 || !SWIGLU), "two to five weight fragments per wave; four with SwiGLU");
+  static_assert(PFD == 0 || FNW == 2 || FNW == 4, "the touch-ahead wants a wave's 64 rows to be of one kind");
   constexpr int BN = 32 * FNW;                          // weight rows of the workgroup
   constexpr int W_BYTES = BN * T_ROWB, STAGE_BYTES = W_BYTES + 128 * T_ROWB;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];   // [stage][w tile, act tile]
@@ -678,13 +683,14 @@ __global__ __launch_bounds__(256, 2) void gemm_pipe_kernel(elem_t* __restrict__ 
 #ifdef VK_BF16
     // Order for the scheduler: the first slab's reads, then the second slab's reads one by one between
     // the first slab's MFMAs, so that they return while the matrix unit works.
+    constexpr int BETWEEN = FNW >= 4 ? 2 : 1;                    // MFMAs between two of the second slab's reads
     __builtin_amdgcn_sched_group_barrier(0x100, FNW + 4, 0);     // the first slab's LDS reads
 #pragma unroll
     for (int q = 0; q < FNW + 4; ++q) {
-      __builtin_amdgcn_sched_group_barrier(0x008, FNW == 4 ? 2 : 1, 0);   // MFMA
+      __builtin_amdgcn_sched_group_barrier(0x008, BETWEEN, 0);            // MFMA
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                  // 1 LDS read
     }
-    __builtin_amdgcn_sched_group_barrier(0x008, FNW == 4 ? 16 : 10, 0);   // the first slab's other MFMAs and the second slab's
+    __builtin_amdgcn_sched_group_barrier(0x008, 8 * FNW - (FNW + 4) * BETWEEN, 0);   // the first slab's other MFMAs and the second slab's
 #endif
   };
   auto close_chunk = [&]() {
@@ -781,7 +787,7 @@ static int launch_pipe(elem_t* out, const elem_t* act, const elem_t* w, int M, i
   dim3 grid((N + BN - 1) / BN, (M + 127) / 128);
   VK_REQUIRE(grid.y <= 65535, "gemm: too many rows (%d)", M);
   const int band_w = (pipe_band_blocks > 0 && grid.y > 1 && (int)grid.x > pipe_band_blocks) ? pipe_band_blocks : (int)grid.x;
-  if constexpr (S == 2) {
+  if constexpr (S == 2 && (FNW == 2 || FNW == 4)) {
     // No more workgroups than compute units: each waits for its own loads with nothing to run meanwhile, and
     // touching the lines four tiles ahead brings them into the second-level cache in time (300 rows, 4,096 x
     // 12,288: 146 -> 112 us).  With more workgroups the touches cost more than they bring: the path from
@@ -1228,14 +1234,43 @@ static int choose_gemm_kernel(int M, int N, int K) {
   return 2;
 }
 
+// How many 16-row weight fragments a wave of the tile kernel takes (a workgroup: 32 of them in weight rows).  The
+// kernel's time goes in rounds of the workgroups that the device holds at once, two per compute unit: a last round
+// that is nearly empty costs almost a whole one (0.72 of one up to half full, where every workgroup has its unit
+// to itself).  A round costs 0.9, 1 and 1.25 times the square tile's with 96, 128 and 160 weight rows (measured at
+// 1,024 to 8,192 rows on 4,096 to 10,240 weight rows); another width is taken when that makes the sum 3 % smaller:
+// 5,120 weight rows at 2,048 rows are 1.25 rounds of 128 or one of 160 (5,120 x 5,120: 121 -> 93 us, 5,120 x
+// 17,408: 452 -> 337, 5,120 x 25,600: 705 -> 481), 6,144 weight rows at 1,024 rows 0.75 rounds of 128 or one of 96
+// (62 -> 53 us).
+static int pipe_fragments_by_rounds(int M, int N) {
+  static const double round_cost[6] = {0, 0, 0, 0.9, 1.0, 1.25};
+  const double slots = 2.0 * device_cus();
+  const int mb = (M + 127) / 128;
+  auto estimate = [&](int f) {
+    const double rounds = (double)((N + 32 * f - 1) / (32 * f)) * mb / slots;
+    const double whole = std::floor(rounds), part = rounds - whole;
+    return round_cost[f] * (whole + (part == 0 ? 0.0 : (part <= 0.5 ? 0.72 : 1.0)));
+  };
+  int best = 4;
+  double least = 0.97 * estimate(4);
+  for (int f : {3, 5}) {
+    const double e = estimate(f);
+    if (e < least) {
+      least = e;
+      best = f;
+    }
+  }
+  return best;
+}
+
 extern "C" {
 
 // kernel: 0 = choose by size, 1 = skinny (M <= 64), 2 = tiled (pipelined if K allows), 3 = tiled through
 // registers, 4..6 = pipelined with 2..4 stages, 7 = skinny with two weight tiles per workgroup where it has
 // such a variant, 8, 9 and 10 = activations shared through LDS with 64, 32 and 128 weight rows per workgroup
 // (17 to 512 rows, in blocks of 64 rows), 11 = skinny with two activation tiles resident in registers (17 to
-// 32 rows of 16-bit elements, K <= 4096), 12 = as 9 in blocks of 32 rows, 13 = pipelined with 64 weight rows
-// per workgroup; for measurements and tests.  The result does not depend on the choice.
+// 32 rows of 16-bit elements, K <= 4096), 12 = as 9 in blocks of 32 rows, 13, 15 and 16 = pipelined with 64, 96
+// and 160 weight rows per workgroup (14 is the callers' name for the route through chunk sums); for measurements and tests.  The result does not depend on the choice.
 int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K, int64_t lda, int64_t ldo,
             int kernel, hipStream_t st) {
   VK_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
@@ -1244,7 +1279,7 @@ int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K
              (long long)lda, VK_VEC);
   VK_REQUIRE(ldo >= N, "gemm: output row stride %lld is smaller than N=%d", (long long)ldo, N);
   VK_REQUIRE(((uintptr_t)act % 16) == 0 && ((uintptr_t)w % 16) == 0, "gemm: operands must be 16-byte aligned");
-  VK_REQUIRE(kernel >= 0 && kernel <= 13, "gemm: unknown kernel %d", kernel);
+  VK_REQUIRE(kernel >= 0 && kernel <= 16 && kernel != 14, "gemm: unknown kernel %d", kernel);
   if (M == 0) return 0;
   const int vec_ok = (ldo % 4 == 0) && ((uintptr_t)out % 16 == 0);
   const bool by_size = kernel == 0;
@@ -1356,6 +1391,9 @@ int vk_gemm(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K
     // compute unit can read, whatever the number of stages).
     const int64_t tiles = (int64_t)((N + 127) / 128) * ((M + 127) / 128);
     if (kernel == 13 || (by_size && tiles <= device_cus())) return launch_pipe<2, false, 2>(out, act, w, M, N, K, lda, ldo, vec_ok, st);
+    const int fragments = kernel == 15 ? 3 : (kernel == 16 ? 5 : (by_size ? pipe_fragments_by_rounds(M, N) : 4));
+    if (fragments == 3) return launch_pipe<2, false, 3>(out, act, w, M, N, K, lda, ldo, vec_ok, st);
+    if (fragments == 5) return launch_pipe<2, false, 5>(out, act, w, M, N, K, lda, ldo, vec_ok, st);
     return launch_pipe<2>(out, act, w, M, N, K, lda, ldo, vec_ok, st);
   }
   return launch_tiled<4, 4>(out, act, w, M, N, K, lda, ldo, vec_ok, st);
