@@ -954,8 +954,8 @@ int vk_attn_prefill_shares_tiles(int d, int P) {
 // items: n_items pairs (sequence, first row).
 // mode 0: each item is up to vk_attn_item_rows() consecutive rows of the sequence's q_len new tokens;
 //   the kernel is chosen by shape.  mode 2: the same through the kernel that takes every shape,
-//   mode 6: through the one that shares tiles in LDS with four waves instead of eight (tests and
-//   measurements; the result is the same bits).
+//   modes 6 and 8: through the one that shares tiles in LDS with four and with eight waves a workgroup,
+//   whatever the shape (tests and measurements; the result is the same bits).
 // mode 1: each item is one token; the keys are split by segment over nseg workgroups (nseg must cover
 //   the longest sequence; scratch must hold vk_attn_scratch_floats(n_items, ...)) and folded by a
 //   second kernel; the kernel is chosen by shape.  modes 3, 4, 5, 7: the same through a named kernel
@@ -971,10 +971,10 @@ int vk_paged_attention(elem_t* out, const elem_t* q, const elem_t* kc, const ele
   VK_REQUIRE(P >= 8 && (P & (P - 1)) == 0, "attention: page size %d must be a power of two >= 8", P);
   VK_REQUIRE(window >= 0, "attention: window %d must not be negative", window);
   VK_REQUIRE(scale > 0.f, "attention: the score scale must be positive");
-  VK_REQUIRE(mode >= 0 && mode <= 7, "attention: unknown mode %d", mode);
-  const int vk_prefill_variant = mode == 6 ? 14 : 0;
+  VK_REQUIRE(mode >= 0 && mode <= 8, "attention: unknown mode %d", mode);
+  const int vk_prefill_variant = mode == 6 ? 14 : (mode == 8 ? 18 : 0);
   const int vk_decode_variant = mode == 3 ? 1 : (mode == 4 ? 2 : (mode == 5 ? 3 : (mode == 7 ? 4 : 0)));
-  if (mode == 6) mode = 0;
+  if (mode == 6 || mode == 8) mode = 0;
   if (mode >= 3) mode = 1;
   if (n_items <= 0) return 0;
   AttnArgs a;
@@ -996,11 +996,13 @@ int vk_paged_attention(elem_t* out, const elem_t* q, const elem_t* kc, const ele
     }                                                                                                \
     attn_prefill_lds_kernel<DP, NW><<<n_items * (ITEM_ROWS / (16 * NW)) * nq, 64 * NW, smem, st>>>(a, n_items); \
   } while (0)
-    // Eight waves of one row tile each measured best on long contexts (MI355X, head size 128); four
-    // waves are a few per cent better on short ones.  Two row tiles per wave would halve the LDS
-    // traffic but need more than the 256 registers that two waves per SIMD leave: with spills or
-    // with one wave per SIMD they measured 40 % slower.
-    const int v = vk_prefill_variant;
+    // Eight waves of one row tile each measured best (MI355X, head size 128) unless they are few: with fewer
+    // workgroups of eight waves than one and a half per compute unit, workgroups of four waves, twice as many,
+    // fill the units better (3 prompts of 300 tokens, 32 heads: 49 -> 43 us; 2 of 1,000 tokens, 8 heads of 64:
+    // 83 -> 74; from two workgroups per unit on eight waves win by 2 to 8 %).  Two row tiles per wave would
+    // halve the LDS traffic but need more than the 256 registers that two waves per SIMD leave: with spills
+    // or with one wave per SIMD they measured 40 % slower.
+    const int v = (vk_prefill_variant == 14 || (vk_prefill_variant == 0 && 2 * (int64_t)n_items * nq < 3 * (int64_t)attn_device_cus())) ? 14 : 0;
     if (d == 64) { if (v == 14) PREFILL_LDS(64, 4); else PREFILL_LDS(64, 8); }
     else if (d == 128) { if (v == 14) PREFILL_LDS(128, 4); else PREFILL_LDS(128, 8); }
     else { if (v == 14) PREFILL_LDS(256, 4); else PREFILL_LDS(256, 8); }
