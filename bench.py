@@ -5,6 +5,7 @@
     python bench.py --shape 0.6b|1.7b|4b|14b|32b    # the same measurement with the layer sizes of another model of the family
     python bench.py --workload mixed14b     # Qwen3-14B shape: 32 prompts of 128 to 4,096 tokens, prefill in portions beside decoding
     python bench.py --workload prefix32b    # Qwen3-32B shape: 64 requests at context 8,192 that share a 1,024-token prefix
+    python bench.py --workload aligned      # the reference's aligned phases: batch 4, cached contexts 0 to 16K, 256 new tokens / 127 decode steps
 
 A step is one decode step of the engine (plan, forward, sample, commit) for a
 batch of B requests whose prompts of 2,048 random tokens were prefilled through
@@ -84,7 +85,7 @@ def main() -> int:
     ap.add_argument("--no-other-shapes", action="store_true", help="skip the 14B and 32B workloads that the default record holds as points")
     ap.add_argument("--prompt-tokens", type=int, default=PROMPT_TOKENS,
                     help="context length of the decode measurement (the prefill figure is always of 2,048 tokens)")
-    ap.add_argument("--workload", default="decode8b", choices=["decode8b", "mixed14b", "prefix32b"])
+    ap.add_argument("--workload", default="decode8b", choices=["decode8b", "mixed14b", "prefix32b", "aligned"])
     ap.add_argument("--engine", default="native", choices=["native", "python"],
                     help="which engine every figure is measured through: the native one (vosti_amd.engine.NativeEngine) or the "
                          "Python step function over the same kernels, cache manager and scheduler")
@@ -104,6 +105,9 @@ def main() -> int:
     from vosti_amd.sampling import SamplingParams
     from vosti_amd.weights import random_weights_on_gpu
 
+    if args.workload == "aligned":
+        print(json.dumps(aligned_workload(args)), flush=True)
+        return 0
     if args.workload != "decode8b":
         print(json.dumps(other_workload(args)), flush=True)
         return 0
@@ -361,6 +365,132 @@ def progress(text: str, state={"t": 0.0}) -> None:
     if now - state["t"] >= 10.0:
         state["t"] = now
         print(f"bench.py: {text}", file=sys.stderr, flush=True)
+
+
+def aligned_workload(args) -> dict:
+    """The reference's controlled phases (scripts/serving_benchmark/aligned/README.md:9-18, 49-53; docs/artifact.md:232-237),
+    through the engine as its own adapter does it (admit all four, then call step): batch 4; cached contexts of 0, 4,096,
+    8,192, 12,288 and 16,384 tokens; a prefill wave adds 256 tokens a request and takes one token (throughput = 1,024
+    new tokens / the median interval of five waves after two untimed ones, an interval being one engine step between two
+    synchronisations); a decode wave times the 127 steps after the first token, every step with the same four requests and
+    replayed from a recorded graph.  To have exactly L tokens cached, an untimed donor of L + 1 tokens that differs from the
+    measured prompt at token L runs first; the engine's count of reused pages must grow by 4 L / 64 in the timed step."""
+    import tempfile
+    import torch
+    from vosti_amd.config import Qwen3Config
+    from vosti_amd.engine import NativeEngine
+    from vosti_amd.sampling import SamplingParams
+
+    if args.engine != "native":
+        raise SystemExit("bench.py: the aligned phases are measured through the native engine")
+    shape = QWEN3_SHAPES[args.shape]
+    layers = args.layers if args.layers is not None else shape["num_hidden_layers"]
+    cfg = Qwen3Config(**dict(shape, num_hidden_layers=layers))
+    elem = 2 if args.dtype == "bfloat16" else 4
+    dt_name = "bf16" if args.dtype == "bfloat16" else "fp32"
+    page, B, new, out_tokens = 64, 4, 256, 128
+    contexts = (0, 4096, 8192, 12288, 16384)
+    model_dir = tempfile.TemporaryDirectory()
+    with open(os.path.join(model_dir.name, "config.json"), "w") as f:
+        json.dump(cfg.to_dict(), f)
+    # Four requests of the longest kind and their donors alive at a time; what earlier waves published stays until the room is wanted.
+    pages = 3 * B * (-(-(contexts[-1] + new + out_tokens + 2) // page)) + 16
+    eng = NativeEngine(model_dir.name, dtype=args.dtype, random_weights_seed=0, num_pages=pages, page_size=page, max_num_seqs=B,
+                       max_num_batched_tokens=4096, enable_prefix_cache=True, graphs=bool(args.graphs))
+    torch.cuda.synchronize()
+    print("bench.py: weights ready", file=sys.stderr, flush=True)
+    rng = random.Random(42)
+    first = iter(range(1000, cfg.vocab_size))          # distinct first tokens across requests and waves
+
+    def tokens(n):
+        return [rng.randrange(cfg.vocab_size) for _ in range(n)]
+
+    def drain():
+        while eng.has_unfinished():
+            eng.step()
+
+    def cohort(L, own):
+        """Four prompts of L cached tokens and `own` new ones; their donors have run and are gone."""
+        prefixes = [[next(first)] + tokens(L - 1) if L else [] for _ in range(B)]
+        if L:
+            for p_ in prefixes:
+                eng.add_request(p_ + [0], SamplingParams(max_tokens=1, ignore_eos=True))      # L + 1 tokens: the pages of the first L are published
+            drain()
+        return [p_ + [next(first)] + tokens(own - 1) for p_ in prefixes]      # token L is not the donor's
+
+    points, detail = {}, {}
+    for L in contexts:
+        # ---- prefill: 256 new tokens a request, one token out ----
+        intervals = []
+        for wave in range(2 + 5):
+            prompts = cohort(L, new)
+            hits = eng.stats()["prefix_hits"]
+            for p_ in prompts:
+                eng.add_request(p_, SamplingParams(max_tokens=1, ignore_eos=True))
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            emitted = eng.step()
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            if len(emitted) != B or eng.has_unfinished():
+                raise RuntimeError(f"aligned prefill at context {L}: the four requests did not run as one step")
+            if eng.stats()["prefix_hits"] - hits != B * (L // page):
+                raise RuntimeError(f"aligned prefill at context {L}: {eng.stats()['prefix_hits'] - hits} pages reused, {B * (L // page)} expected")
+            if wave >= 2:
+                intervals.append(dt)
+        intervals.sort()
+        med = intervals[len(intervals) // 2]
+        points[f"prefill_ctx{L}"] = round(B * new / med, 1)
+        detail[f"prefill_ctx{L}_ms"] = [round(x * 1e3, 3) for x in intervals]
+        progress(f"aligned: context {L}: prefill {points[f'prefill_ctx{L}']} tok/s")
+        # ---- decode: one new token a request, then 127 timed steps ----
+        rates = []
+        for wave in range(1 + 2):
+            prompts = cohort(L, 1)
+            for p_ in prompts:
+                eng.add_request(p_, SamplingParams(max_tokens=out_tokens, ignore_eos=True))
+            if len(eng.step()) != B:                   # the first token of each: outside the timing
+                raise RuntimeError(f"aligned decode at context {L}: the first step did not emit for all four")
+            before = eng.stats()["graph_stats"]
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(out_tokens - 1):
+                if len(eng.step()) != B:
+                    raise RuntimeError(f"aligned decode at context {L}: a step did not emit for all four")
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            after = eng.stats()["graph_stats"]
+            if eng.has_unfinished():
+                raise RuntimeError("aligned decode: requests left after 128 tokens")
+            replayed_only = after["eager"] == before["eager"] and after["captured"] == before["captured"]
+            if wave >= 1:
+                if args.graphs and not replayed_only:
+                    raise RuntimeError(f"aligned decode at context {L}: a timed step was recorded or ran eagerly")
+                rates.append(B * (out_tokens - 1) / dt)
+        rates.sort()
+        points[f"decode_ctx{L}"] = round(rates[len(rates) // 2], 1)
+        progress(f"aligned: context {L}: decode {points[f'decode_ctx{L}']} tok/s")
+    name = f"Qwen3-{args.shape.upper()} shape"
+    layers_w, head_w = gemm_params(cfg)
+    kv_token = 2 * cfg.num_key_value_heads * cfg.head_dim * cfg.num_hidden_layers
+    step_s = B / points["decode_ctx4096"]
+    read = (layers_w + head_w + B * (4096 + 1 + out_tokens / 2) * kv_token) * elem
+    flops4k = 2.0 * B * new * layers_w + 2.0 * B * head_w + 4.0 * cfg.num_attention_heads * cfg.head_dim * B * new * (4096 + new / 2) * cfg.num_hidden_layers
+    t4k = B * new / points["prefill_ctx4096"]
+    return {"metric": f"aligned phases at batch 4 (the reference's method): decode tok/s over 127 steps at cached context 4,096, {name}",
+            "value": points["decode_ctx4096"], "unit": "tokens/s", "n_gpus": 1, "steps": out_tokens - 1, "warmup": 1,
+            "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dt_name,
+            "data": "synthetic: seeded random token prompts (seed 42), seeded random weights",
+            "config": {"model": name, "layers": layers, "layers_of_model": shape["num_hidden_layers"], "hidden_size": cfg.hidden_size,
+                       "intermediate_size": cfg.intermediate_size, "q_heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
+                       "head_dim": cfg.head_dim, "vocab_size": cfg.vocab_size, "global_batch": B, "new_prefill_tokens": new,
+                       "output_tokens": out_tokens, "page_size": page, "parallelism": "single GPU", "graphs": bool(args.graphs),
+                       "engine": "native", "prefill_waves": "2 untimed + 5", "decode_waves": "1 untimed + 2"},
+            "prefill": {"value": points["prefill_ctx4096"], "tokens": B * new, "ms": round(t4k * 1e3, 3),
+                        "frac": round(flops4k / t4k / PEAK_FLOPS[dt_name], 4), "cached_context": 4096},
+            "roofline": {"bound": "hbm", "achieved": round(read / step_s / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(read / step_s / 1e9 / HBM_PEAK_GBS, 4)},
+            "points": points, "intervals": detail}
 
 
 def other_workload(args) -> dict:
