@@ -396,7 +396,7 @@ def test_attention_prompt_kernels_agree(dtype, nq, nkv, d, P, window):
         kk.append(rand((kl, nkv, d), dtype, 30 + i))
         vv.append(rand((kl, nkv, d), dtype, 50 + i))
     got = run_attention(k, q_list, kk, vv, P, dtype, window=window, poison=float("nan"))
-    for mode in (2, 6, 8):     # the kernel for every shape, and shared tiles with four and with eight waves a workgroup
+    for mode in (2, 6, 8, 9):  # the kernel for every shape, and shared tiles with four waves, eight, and four with one buffer
         if mode != 2 and not k.lib.vk_attn_prefill_shares_tiles(d, P):
             continue
         other = run_attention(k, q_list, kk, vv, P, dtype, window=window, poison=float("nan"), seed=3, prompt_mode=mode)
@@ -496,7 +496,7 @@ def test_attention_far_key_in_prompt_rows(dtype):
         q[:, :, 0] = 40.0
         kx[far, :, 0] = 40.0
         want = vx[far].float().repeat_interleave(nq // nkv, dim=0)
-        for mode in (0, 2, 6, 8):      # by shape, the kernel for every shape, shared tiles with four and with eight waves
+        for mode in (0, 2, 6, 8, 9):   # by shape, the kernel for every shape, shared tiles with four waves, eight, four and one buffer
             got = run_attention(k, [q], [kx], [vx], P, dtype, prompt_mode=mode)
             first = max(0, far - (L - n))          # the first row of the portion that sees the key
             torch.testing.assert_close(got[first:].float(), want.expand(n - first, -1, -1), **tol(dtype))

@@ -442,7 +442,7 @@ __device__ __forceinline__ int key_swz(int row) { return row & 15; }
 __device__ __forceinline__ int val_swz(int row) { return row & 15; }          // rows of 256 bytes
 #endif
 
-template <int DPAD, int NW>
+template <int DPAD, int NW, int NST = 2>
 __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_lds_kernel(AttnArgs a, int n_items) {
   constexpr int ROWS_WG = 16 * NW;                       // NW waves, each with one 16-row tile
   constexpr int BPI = ITEM_ROWS / ROWS_WG;               // workgroups per item
@@ -540,10 +540,10 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_lds_kernel(AttnArgs a
 
   issue(tile_lo, 0);
   for (int t = tile_lo; t <= tile_hi; ++t) {
-    const int stage = (t - tile_lo) & 1;
+    const int stage = NST == 2 ? (t - tile_lo) & 1 : 0;
     wait_vm_loads();
     __syncthreads();      // tile t is in LDS; every wave is done with the other buffer
-    if (t < tile_hi) issue(t + 1, stage ^ 1);
+    if (NST == 2 && t < tile_hi) issue(t + 1, stage ^ 1);
     if (t * TILE_KEYS + TILE_KEYS > k_len || t * TILE_KEYS < item_lo) {
       // Keys outside [item_lo, k_len) may lie in pages this sequence does not own: their values are replaced by
       // zero in LDS, so that stale NaN or Inf cannot reach a sum (their probabilities are zero).  The first and
@@ -607,6 +607,10 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_lds_kernel(AttnArgs a
         for (int ks = 0; ks < KEY_SLABS; ++ks) As[dt] = mma_slab(vf[ks], pf[ks], As[dt]);
       }
       __builtin_amdgcn_s_setprio(0);
+    }
+    if (NST == 1 && t < tile_hi) {                         // one buffer: the next tile may come when every wave has read this one
+      __syncthreads();
+      issue(t + 1, 0);
     }
     if ((t + 1) % SEG_TILES == 0 || t == tile_hi) {        // the segment is complete
       fold<NDT>(M, L, ACC, Ms, Ls, As);
@@ -954,8 +958,8 @@ int vk_attn_prefill_shares_tiles(int d, int P) {
 // items: n_items pairs (sequence, first row).
 // mode 0: each item is up to vk_attn_item_rows() consecutive rows of the sequence's q_len new tokens;
 //   the kernel is chosen by shape.  mode 2: the same through the kernel that takes every shape,
-//   modes 6 and 8: through the one that shares tiles in LDS with four and with eight waves a workgroup,
-//   whatever the shape (tests and measurements; the result is the same bits).
+//   modes 6, 8 and 9: through the one that shares tiles in LDS with four waves, with eight, and with four and
+//   one buffer instead of two, whatever the shape (tests and measurements; the result is the same bits).
 // mode 1: each item is one token; the keys are split by segment over nseg workgroups (nseg must cover
 //   the longest sequence; scratch must hold vk_attn_scratch_floats(n_items, ...)) and folded by a
 //   second kernel; the kernel is chosen by shape.  modes 3, 4, 5, 7: the same through a named kernel
@@ -971,10 +975,10 @@ int vk_paged_attention(elem_t* out, const elem_t* q, const elem_t* kc, const ele
   VK_REQUIRE(P >= 8 && (P & (P - 1)) == 0, "attention: page size %d must be a power of two >= 8", P);
   VK_REQUIRE(window >= 0, "attention: window %d must not be negative", window);
   VK_REQUIRE(scale > 0.f, "attention: the score scale must be positive");
-  VK_REQUIRE(mode >= 0 && mode <= 8, "attention: unknown mode %d", mode);
-  const int vk_prefill_variant = mode == 6 ? 14 : (mode == 8 ? 18 : 0);
+  VK_REQUIRE(mode >= 0 && mode <= 9, "attention: unknown mode %d", mode);
+  const int vk_prefill_variant = mode == 6 ? 14 : (mode == 8 ? 18 : (mode == 9 ? 19 : 0));
   const int vk_decode_variant = mode == 3 ? 1 : (mode == 4 ? 2 : (mode == 5 ? 3 : (mode == 7 ? 4 : 0)));
-  if (mode == 6 || mode == 8) mode = 0;
+  if (mode == 6 || mode == 8 || mode == 9) mode = 0;
   if (mode >= 3) mode = 1;
   if (n_items <= 0) return 0;
   AttnArgs a;
@@ -996,6 +1000,16 @@ int vk_paged_attention(elem_t* out, const elem_t* q, const elem_t* kc, const ele
     }                                                                                                \
     attn_prefill_lds_kernel<DP, NW><<<n_items * (ITEM_ROWS / (16 * NW)) * nq, 64 * NW, smem, st>>>(a, n_items); \
   } while (0)
+#define PREFILL_LDS1(DP)                                                                             \
+  do {                                                                                               \
+    static bool raised = false;                                                                      \
+    if (!raised) {                                                                                   \
+      (void)hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<DP, 4, 1>,                      \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);              \
+      raised = true;                                                                                 \
+    }                                                                                                \
+    attn_prefill_lds_kernel<DP, 4, 1><<<n_items * (ITEM_ROWS / 64) * nq, 256, smem / 2, st>>>(a, n_items); \
+  } while (0)
     // Eight waves of one row tile each measured best (MI355X, head size 128) unless they are few: with fewer
     // workgroups of eight waves than one and a half per compute unit, workgroups of four waves, twice as many,
     // fill the units better (3 prompts of 300 tokens, 32 heads: 49 -> 43 us; 2 of 1,000 tokens, 8 heads of 64:
@@ -1003,10 +1017,21 @@ int vk_paged_attention(elem_t* out, const elem_t* q, const elem_t* kc, const ele
     // halve the LDS traffic but need more than the 256 registers that two waves per SIMD leave: with spills
     // or with one wave per SIMD they measured 40 % slower.
     const int v = (vk_prefill_variant == 14 || (vk_prefill_variant == 0 && 2 * (int64_t)n_items * nq < 3 * (int64_t)attn_device_cus())) ? 14 : 0;
+    // With many workgroups (two rounds or more of the three four-wave workgroups that a compute unit holds when
+    // each has one buffer of 32 KB) the occupancy is worth more than loads that overlap a workgroup's own work:
+    // 12 waves a unit instead of 8 (2 prompts of 2,048 tokens: 140 -> 121 us; 8,192 tokens: 890 -> 718, with 64
+    // heads 1,580 -> 1,388).  With fewer it loses to the rounds (2,048 rows after 14,336 keys: 756 -> 825).
+    const bool one_buffer = vk_prefill_variant == 19 ||
+                            (vk_prefill_variant == 0 && sizeof(elem_t) == 2 && (int64_t)n_items * nq >= 3 * (int64_t)attn_device_cus());
+    if (one_buffer) {
+      if (d == 64) PREFILL_LDS1(64); else if (d == 128) PREFILL_LDS1(128); else PREFILL_LDS1(256);
+      return vk_check_launch("attention (prompt rows, shared tiles, one buffer)");
+    }
     if (d == 64) { if (v == 14) PREFILL_LDS(64, 4); else PREFILL_LDS(64, 8); }
     else if (d == 128) { if (v == 14) PREFILL_LDS(128, 4); else PREFILL_LDS(128, 8); }
     else { if (v == 14) PREFILL_LDS(256, 4); else PREFILL_LDS(256, 8); }
 #undef PREFILL_LDS
+#undef PREFILL_LDS1
     return vk_check_launch("attention (prompt rows, shared tiles)");
   }
   if (mode != 1) {

@@ -333,7 +333,7 @@ class Kernels:
         """Attention of the rows named by ``items`` over the paged cache (see attention.hip).
 
         items [n, 2] = (sequence, first row).  mode 0: an item is up to ATTN_ITEM_ROWS consecutive new
-        rows of its sequence; modes 2, 6 and 8: the same through a named kernel (same bits); mode 1: an item
+        rows of its sequence; modes 2, 6, 8 and 9: the same through a named kernel (same bits); mode 1: an item
         is a single decoded token; modes 3, 4, 5, 7: the same through a named kernel (same bits; see
         attention.hip).  ``max_k_len`` is the host's bound on k_len; the block table must cover it."""
         T, nq, d = q.shape
