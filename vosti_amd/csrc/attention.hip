@@ -539,8 +539,10 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_lds_kernel(AttnArgs a
   for (int dt = 0; dt < NDT; ++dt) ACC[dt] = As[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   issue(tile_lo, 0);
-  for (int t = tile_lo; t <= tile_hi; ++t) {
-    const int stage = NST == 2 ? (t - tile_lo) & 1 : 0;
+  // The buffer a tile lies in is a constant in the code of its step (the loop below takes two steps a turn), so that
+  // the LDS addresses of the fragments are computed once for the kernel and not added to a buffer's base in every tile.
+  auto step = [&](int t, auto stage_c) {
+    constexpr int stage = decltype(stage_c)::value;
     wait_vm_loads();
     __syncthreads();      // tile t is in LDS; every wave is done with the other buffer
     if (NST == 2 && t < tile_hi) issue(t + 1, stage ^ 1);
@@ -619,6 +621,10 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_lds_kernel(AttnArgs a
 #pragma unroll
       for (int dt = 0; dt < NDT; ++dt) As[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
+  };
+  for (int t = tile_lo; t <= tile_hi; t += 2) {
+    step(t, std::integral_constant<int, 0>{});
+    if (t + 1 <= tile_hi) step(t + 1, std::integral_constant<int, NST == 2 ? 1 : 0>{});
   }
   if (row_ok) {
     const float inv = L > 0.f ? 1.0f / L : 0.f;
