@@ -278,6 +278,53 @@ def test_qkv_post(dtype, nq, nkv, d, P, rot):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,d,P", [(4, 2, 64, 16), (8, 2, 128, 64), (2, 1, 256, 8), (3, 3, 128, 32)])
+def test_cache_store_of_a_long_step(dtype, nq, nkv, d, P):
+    """A step of many tokens takes other launch shapes than a step of few (all heads of a token per workgroup).
+    The rows here are decoded tokens with scattered slots, a portion that begins at a page's first place but at
+    row 5 of the step, a portion that begins in the middle of a page, rows that store nothing, and a short tail:
+    both caches must hold exactly what storing the rows nine at a time leaves, every value row is the input row
+    bytewise, and nothing else is touched."""
+    k = kern(dtype)
+    n_pages, eps = 40, 1e-6
+    g = torch.Generator().manual_seed(5)
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    slots = [perm[0] * P + 3, perm[1] * P + P - 1, -1, perm[2] * P, perm[3] * P + 5]            # decoded tokens
+    run = lambda page_list, first, n: [page_list[(first + i) // P] * P + (first + i) % P for i in range(n)]
+    slots += run(perm[4:16], 0, 77)                    # begins at a page's first place, at row 5
+    slots += [-1, -1, -1]
+    slots += run(perm[16:26], 13, 50)                  # begins inside a page
+    slots += run(perm[26:30], 8, 11)                   # an aligned beginning, too short for a second run
+    slots[40] = -1                                     # a hole inside a run
+    T = len(slots)
+    assert T >= 64 and len(set(x for x in slots if x >= 0)) == len([x for x in slots if x >= 0])
+    qkv = rand((T, (nq + 2 * nkv) * d), dtype, 1)
+    qw, kw = (1 + 0.1 * rand((d,), torch.float32, 2)).to(dtype), (1 + 0.1 * rand((d,), torch.float32, 3)).to(dtype)
+    positions = torch.arange(T, dtype=torch.int32)
+    inv = (1.0 / (1e4 ** (torch.arange(0, d, 2, dtype=torch.int64).float() / d))).cuda()
+    cos, sin = k.rope_tables(inv, T + 1)
+    st = torch.tensor(slots, dtype=torch.int32)
+
+    def store(rows):
+        kc = torch.full((n_pages, nkv, P, d), 7.0, dtype=dtype).cuda()
+        vc = torch.full((n_pages, nkv, d, P), 7.0, dtype=dtype).cuda()
+        qs = [k.qkv_post(qkv[a:b].cuda(), nq=nq, nkv=nkv, d=d, q_out=None, k_cache=kc, v_cache=vc, page_size=P, q_w=qw.cuda(), k_w=kw.cuda(),
+                         eps=eps, cos=cos, sin=sin, positions=positions[a:b].cuda(), slots=st[a:b].cuda()) for a, b in rows]
+        return torch.cat(qs).cpu(), kc.cpu(), vc.cpu()
+
+    q_all, kc_all, vc_all = store([(0, T)])
+    q_one, kc_one, vc_one = store([(t, min(t + 9, T)) for t in range(0, T, 9)])      # nine rows a call: the launch shape of few tokens
+    assert torch.equal(q_all, q_one) and torch.equal(kc_all, kc_one) and torch.equal(vc_all, vc_one)
+    x = qkv.view(T, nq + 2 * nkv, d)
+    written = torch.zeros(n_pages * P, dtype=torch.bool)
+    for t, s_ in enumerate(slots):
+        if s_ >= 0:
+            written[s_] = True
+            assert torch.equal(vc_all[s_ // P, :, :, s_ % P], x[t, nq + nkv:]), (t, s_)
+    assert (vc_all.permute(0, 3, 1, 2).reshape(n_pages * P, nkv, d)[~written] == 7.0).all()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_rope_invariants(dtype):
     """Position 0 is the identity; a rotation keeps each pair's norm; the product of a
     rotated q and k depends on the distance of their positions only (float32)."""
