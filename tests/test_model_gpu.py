@@ -222,11 +222,14 @@ def test_trace_run_program(tiny_dirs, plain_logits, tmp_path, dtype_name):
         {"step": 0, "entries": [{"id": "a", "tokens": prompts[a][:40], "want": [0, 39]}], "end": []},
         {"step": 1, "entries": [{"id": "a", "tokens": prompts[a][40:], "want": [24]},
                                 {"id": "b", "tokens": prompts[b][:100], "want": []}], "end": ["a"]},
-        {"step": 2, "entries": [{"id": "b", "tokens": prompts[b][100:128], "want": [27]}], "end": []},
+        {"step": 9, "entries": [], "end": []},                      # a step that brings nothing: answered, no file
+        {"step": 2, "entries": [{"id": "b", "tokens": prompts[b][100:128], "want": [27]},
+                                {"id": "idle", "tokens": [], "want": []}], "end": ["never seen"]},      # an entry without tokens is as good as left out
         {"step": 3, "entries": [{"id": "b", "tokens": prompts[b][128:], "want": [0]}], "end": ["b"]},
         {"step": 4, "entries": [{"id": "c", "tokens": prompts[c], "want": [119]}], "end": ["c"]},
     ]
     run_trace(tiny_dirs[name], dtype_name, tmp_path, max_tokens=128 + 192, steps=steps)
+    assert not (tmp_path / "9.f32").exists()
     read = lambda s, d=tmp_path: torch.from_numpy(np.fromfile(d / f"{s}.f32", dtype="<f4").reshape(-1, vocab))
     # The few rows that were asked for, against the same rows of the plain logits.
     got = torch.cat([read(s) for s in range(5)])

@@ -93,6 +93,11 @@ def main(argv: list[str] | None = None) -> int:
         entries = []
         for e in rec.get("entries", []):
             name = str(e["id"])
+            if not e.get("tokens"):
+                # Nothing to run for this request in this step: the same as leaving it out.
+                if e.get("want"):
+                    raise SystemExit(f"trace_run: step {step}: request {name} asks for logits but brings no tokens")
+                continue
             if name not in ids:
                 ids[name] = next_id
                 next_id += 1
@@ -113,7 +118,7 @@ def main(argv: list[str] | None = None) -> int:
             entries.append((ids[name], [int(t) for t in e["tokens"]], [int(w) for w in e.get("want", [])]))
         # Which row of the step's file is which: [request id, position of the token in the request] per wanted place.
         index = []
-        for e, (rid, tokens, want) in zip(rec.get("entries", []), entries):
+        for e, (rid, tokens, want) in zip([e for e in rec.get("entries", []) if e.get("tokens")], entries):
             name = str(e["id"])
             index += [[e["id"], fed.get(name, 0) + w] for w in want]
             fed[name] = fed.get(name, 0) + len(tokens)
