@@ -223,6 +223,29 @@ def main() -> int:
                              "frac": round(flops / t / PEAK_FLOPS[dt_name], 4), "of": "median of six", "best_ms": round(times[0] * 1e3, 3),
                              "engine": args.engine}
         points = {}
+        other_shapes = not args.no_other_shapes and args.shape == "8b" and args.dtype == "bfloat16"
+
+        def other_point(workload):
+            """One of the two larger workloads of the same family, whole models, as points of this record (their own
+            records: --workload mixed14b, --workload prefix32b)."""
+            other_args = argparse.Namespace(**dict(vars(args), workload=workload, layers=None, batch=None, steps=16, warmup=8))
+            try:
+                r = other_workload(other_args)
+            except Exception as e:          # the record's own figures stand without these
+                points[workload + "_error"] = f"{type(e).__name__}: {e}"
+                return
+            if workload == "mixed14b":
+                points.update(mixed14b_tokens_per_s=r["value"], mixed14b_output_tokens_per_s=r["output"]["value"],
+                              mixed14b_wall_s=r["output"]["wall_s"])
+            else:
+                points.update(prefix32b_decode_b64_tokens_per_s=r["value"], prefix32b_ms_per_step=r["ms_per_step"],
+                              prefix32b_roofline_frac=r["roofline"]["frac"], prefix32b_prefill_tokens_per_s=r["prefill"]["value"])
+
+        # The mixed workload is a few seconds of matrix work, and the card's clock drops for a while after a long
+        # stretch of that (the same workload right after the batch 64 prompts and the kernels' own timing: 16 k
+        # tokens a second instead of 21 k): it runs here, while little such work lies behind.
+        if other_shapes:
+            other_point("mixed14b")
         # At batch 1 the first forty or so steps after a new engine's prompt run 4 % slower than the rest (4.35 against
         # 4.18 ms), whichever engine runs them: the point is taken after 48 untimed steps, and the steps right after
         # the prompt and those after 150 steps stand beside it.
@@ -243,24 +266,10 @@ def main() -> int:
                 kernels["prefill"] = {"error": f"{type(e).__name__}: {e}"}
     if kernels:
         record["kernels"] = kernels
-    if not args.no_points and not args.no_other_shapes and args.shape == "8b" and args.dtype == "bfloat16":
-        # The two larger workloads of the same family, whole models, as points of this record (their own records:
-        # --workload mixed14b, --workload prefix32b).
+    if not args.no_points and other_shapes:
         del model
         torch.cuda.empty_cache()
-        for workload in ("mixed14b", "prefix32b"):
-            other_args = argparse.Namespace(**dict(vars(args), workload=workload, layers=None, batch=None, steps=16, warmup=8))
-            try:
-                r = other_workload(other_args)
-            except Exception as e:          # the record's own figures stand without these
-                record["points"][workload + "_error"] = f"{type(e).__name__}: {e}"
-                continue
-            if workload == "mixed14b":
-                record["points"].update(mixed14b_tokens_per_s=r["value"], mixed14b_output_tokens_per_s=r["output"]["value"],
-                                        mixed14b_wall_s=r["output"]["wall_s"])
-            else:
-                record["points"].update(prefix32b_decode_b64_tokens_per_s=r["value"], prefix32b_ms_per_step=r["ms_per_step"],
-                                        prefix32b_roofline_frac=r["roofline"]["frac"], prefix32b_prefill_tokens_per_s=r["prefill"]["value"])
+        other_point("prefix32b")            # last: its prompts alone are half a minute of matrix work
     print(json.dumps(record), flush=True)
     return 0
 
